@@ -86,11 +86,12 @@ class ModelConfig:
     linear_value_head_dim: int = 0
     linear_conv_kernel_dim: int = 4
 
-    # -- per-layer stacks (vurizen, sogidra): every layer carries its own mixer and
+    # -- per-layer stacks (vurizen, sogidra, zabusun): every layer carries its own mixer and
     # feed-forward description; the flat fields above hold the first layer's
     # values only so that sizing helpers have something to read ----------------
     layer_specs: Optional[List[Dict[str, Any]]] = None
     residual_mult: float = 1.0
+    logit_scale: float = 1.0         # the logits are multiplied by this
 
     raw: Dict[str, Any] = field(default_factory=dict, repr=False)
 
@@ -129,6 +130,11 @@ class ModelConfig:
                 elif sp["type"] == "attention_2":    # values = unnormed keys
                     g = int(mx.get("kv_heads", mx["heads"]))
                     dims.append((g * int(mx["dim"]), g * int(mx["dim"])))
+                elif sp["type"] == "parallel":       # the attention half's rows
+                    left = mx["left"]
+                    g = int(left.get("kv_heads", left["heads"]))
+                    dims.append((g * int(left["dim"]),
+                                 g * int(left.get("vdim", left["dim"]))))
             return dims
         if not self.is_mla:
             return []
@@ -145,7 +151,7 @@ class ModelConfig:
             mx = sp["mixer"]
             if mx.get("kv_from") is not None:
                 continue
-            if sp["type"] in ("latent_attention", "attention"):
+            if sp["type"] in ("latent_attention", "attention", "parallel"):
                 out.append(0)
             elif sp["type"] == "attention_2":
                 out.append(int((mx.get("mask") or {}).get("pool", 0)))
@@ -155,11 +161,15 @@ class ModelConfig:
         """(conv-state shape, recurrent-state shape) of every linear-attention
         layer in [start, end)."""
         if self.layer_specs is not None:
-            return [
-                ((0,), (int(sp["mixer"]["heads"]), int(sp["mixer"]["dim"]),
-                        int(sp["mixer"]["vdim"])))
-                for sp in self.layer_specs[start:end] if sp["type"] == "gla"
-            ]
+            shapes = []
+            for sp in self.layer_specs[start:end]:
+                mx = sp["mixer"]
+                if sp["type"] == "gla":
+                    shapes.append(((0,), (int(mx["heads"]), int(mx["dim"]),
+                                          int(mx["vdim"]))))
+                elif sp["type"] == "parallel":   # the recurrent half: a vector
+                    shapes.append(((0,), (int(mx["right"]["width"]),)))
+            return shapes
         if not self.has_linear_layers:
             return []
         conv_dim = (2 * self.linear_num_key_heads * self.linear_key_head_dim
@@ -180,6 +190,9 @@ class ModelConfig:
 
     @property
     def has_linear_layers(self) -> bool:
+        """Whether any layer keeps recurrent state in a per-request slot."""
+        if self.layer_specs is not None:
+            return any(sp["type"] in ("gla", "parallel") for sp in self.layer_specs)
         return bool(self.layer_types) and "linear_attention" in self.layer_types
 
     def layer_type(self, layer_idx: int) -> str:
@@ -208,11 +221,14 @@ class ModelConfig:
         "norm": {"eps"}, "vocab", "width", ...}). Mixer types: 'gla',
         'latent_attention' (vurizen); 'attention' (differential softmax
         attention), 'attention_2' (sliding window with pooled blocks)
-        (sogidra). Feed-forward kinds: 'moe' (default), 'dense'."""
+        (sogidra); 'parallel' (sigmoid attention beside a minGRU, both reading
+        the layer's input) (zabusun). Feed-forward kinds: 'moe' (default),
+        'dense'."""
         layers = cfg["layers"]
         kinds = {"gla": "linear_attention", "latent_attention": "latent_attention",
                  "attention": "diff_attention",
-                 "attention_2": "pooled_window_attention"}
+                 "attention_2": "pooled_window_attention",
+                 "parallel": "parallel_attention_recurrent"}
         for sp in layers:
             if sp["type"] not in kinds:
                 raise ValueError(f"unknown layer type {sp['type']!r}")
@@ -230,6 +246,8 @@ class ModelConfig:
         moes = [m for m in mlps if kind_of(m) == "moe"]
         dense = [m for m in mlps if kind_of(m) == "dense"]
         first = layers[0]["mixer"]
+        if layers[0]["type"] == "parallel":
+            first = first["left"]
         mc = cls(
             architecture=cfg["architecture"],
             model_type=str(cfg["architecture"]).lower(),
@@ -247,6 +265,7 @@ class ModelConfig:
             torch_dtype=cfg.get("torch_dtype", "bfloat16"),
             layer_specs=layers,
             residual_mult=float(cfg.get("residual_mult", 1.0)),
+            logit_scale=float(cfg.get("logit_scale", 1.0)),
             raw=cfg,
         )
         if latent:

@@ -1,4 +1,7 @@
-"""Gated linear attention (GLA): a matrix-valued recurrent state per head with
+"""Recurrent sequence mixers whose state lives in the engine's per-request
+slots: gated linear attention (below) and minGRU (class MinGRU).
+
+Gated linear attention (GLA): a matrix-valued recurrent state per head with
 a data-dependent decay per key channel,
 
     S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,     o_t = S_t^T (q_t / sqrt(dk)),
@@ -62,3 +65,51 @@ class GatedLinearAttention(nn.Module):
         )
         return self.o_proj(ops.gated_rmsnorm(o, g, self.norm_weight, self.eps,
                                              x.dtype))
+
+
+class MinGRU(nn.Module):
+    """minGRU: a gated recurrence over a vector state whose gates read only
+    the current token, so the whole portion's gate pre-activations come from
+    one GEMM and the recurrence itself is elementwise,
+
+        z_t = sigmoid(W_z h_t + b_z),   u_t = W_x h_t + b_x,
+        c_t = u_t + 1/2 (u_t >= 0)  |  sigmoid(u_t) (u_t < 0),
+        S_t = (1 - z_t) S_(t-1) + z_t c_t,      o_t = S_t * silu(W_g h_t),
+
+    followed by the output projection. The state [width] lives in the
+    engine's LinearStateCache slots in fp32; gates, candidate and state are
+    fp32 whatever the activation dtype. Prompt portions and decode steps run
+    the same kernel (ops.mingru_scan), token-serial per channel.
+
+    own_proj False: the module has no input projection of its own; a caller
+    that merges it with other projections of the same input hands the
+    pre-activations [z | u | g] (`proj_sizes` wide) to mix()."""
+
+    def __init__(self, hidden_size: int, width: int, state_layer_idx: int,
+                 own_proj: bool = True):
+        super().__init__()
+        self.width = int(width)
+        self.state_layer_idx = state_layer_idx
+        self.proj_sizes = [self.width] * 3       # z | u | g
+        self.in_proj = MergedColumnParallelLinear(hidden_size, self.proj_sizes) \
+            if own_proj else None
+        self.z_bias = nn.Parameter(torch.empty(self.width), requires_grad=False)
+        self.x_bias = nn.Parameter(torch.empty(self.width), requires_grad=False)
+        self.o_proj = RowParallelLinear(self.width, hidden_size)
+        self._b32 = None
+
+    def invalidate_constants(self) -> None:
+        self._b32 = None
+
+    def mix(self, zug: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        """zug [T, 3 * width] (a strided view is fine) -> S_t * silu(g_t)."""
+        if self._b32 is None or self._b32[0].device != zug.device:
+            self._b32 = (self.z_bias.detach().float().contiguous(),
+                         self.x_bias.detach().float().contiguous())
+        state = meta.linear_cache.recurrent_states[self.state_layer_idx]
+        return ops.mingru_scan(zug, self._b32[0], self._b32[1], state,
+                               meta.linear_slots, meta.query_bounds(),
+                               meta.positions, self.o_proj.weight.dtype)
+
+    def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        return self.o_proj(self.mix(self.in_proj(x), meta))

@@ -118,6 +118,16 @@ class FusedMoE(nn.Module):
         # stacks that add the expert sum into an fp32 residual take the
         # kernel's fp32 accumulator as it is
         self.fp32_output = False
+        # True: the routing weight multiplies the expert's INPUT, out =
+        # sum_k expert_k(w_k x), instead of its output. Gate and up
+        # projections are linear, so the kernels scale their fp32
+        # accumulators by w_k before the activation.
+        self.weight_on_input = False
+
+    @staticmethod
+    def grouped_kernel_fits(hidden: int, inter: int, fp8: bool = False) -> bool:
+        """Whether the grouped-GEMM kernels tile these sizes."""
+        return hidden % 32 == 0 and inter % (64 if fp8 else 32) == 0
 
     def enable_routing_stats(self) -> None:
         self.routing_counts = torch.zeros(
@@ -212,11 +222,15 @@ class FusedMoE(nn.Module):
                 valid, local, torch.full_like(local, self.num_local_experts)
             )
             topk_w = topk_w * valid
-        # the grouped-GEMM kernels take bf16 activations and tile H by 32 and
-        # I by 64; other types and sizes run the per-expert loop below
-        if x.is_cuda and x.dtype == torch.bfloat16 and H % 32 == 0 \
-                and self.intermediate_size % 64 == 0:
+        # the grouped-GEMM kernels take bf16 activations and tile H and I by
+        # 32 (the fp8 ones I by 64); other types and sizes run the per-expert
+        # loop below
+        if x.is_cuda and x.dtype == torch.bfloat16 and self.grouped_kernel_fits(
+                H, self.intermediate_size, self.fp8):
             if self.fp8:
+                if self.weight_on_input:
+                    raise NotImplementedError(
+                        "fp8 experts with the routing weight on the input")
                 out = ops.fused_moe_forward_fp8(
                     x, self.w_gate_up_fp8, self.w_gu_scale,
                     self.w_down_fp8, self.w_down_scale, topk_ids, topk_w,
@@ -226,6 +240,7 @@ class FusedMoE(nn.Module):
                 out = ops.fused_moe_forward(
                     x, self.w_gate_up, self.w_down, topk_ids, topk_w,
                     limit=self.act_limit,
+                    weight_on_input=self.weight_on_input,
                 )
             if self.ep_size > 1:
                 out = self._comm.tp_all_reduce(out)
@@ -244,18 +259,23 @@ class FusedMoE(nn.Module):
             toks = token_idx[sel]
             xe = x[toks]                              # [n_e, H]
             h = F.linear(xe, self._expert_gu(e, xe.dtype))  # [n_e, 2I]
+            if self.weight_on_input:
+                # fp32 from the scaling to the activation's result
+                h = h.float() * flat_w[sel].unsqueeze(-1)
             if self.act_limit > 0:
                 I = self.intermediate_size
                 gate = h[:, :I].clamp(max=self.act_limit)
                 up = h[:, I:].clamp(min=-self.act_limit, max=self.act_limit)
-                h = (up + 1.0) * (gate * torch.sigmoid(gate * 1.702))
-            elif h.is_cuda and h.dtype != torch.bfloat16:
+                h = ((up + 1.0) * (gate * torch.sigmoid(gate * 1.702))).to(xe.dtype)
+            elif (h.is_cuda and h.dtype != torch.bfloat16) or self.weight_on_input:
                 I = self.intermediate_size
-                h = F.silu(h[:, :I]) * h[:, I:]
+                h = (F.silu(h[:, :I]) * h[:, I:]).to(xe.dtype)
             else:
                 h = ops.silu_and_mul(h)
             ye = F.linear(h, self._expert_down(e, h.dtype)).float()  # [n_e, H]
-            out.index_add_(0, toks, ye * flat_w[sel].unsqueeze(-1))
+            if not self.weight_on_input:
+                ye = ye * flat_w[sel].unsqueeze(-1)
+            out.index_add_(0, toks, ye)
         if self.ep_size > 1:
             out = self._comm.tp_all_reduce(out)
         return out if self.fp32_output else out.to(x.dtype)

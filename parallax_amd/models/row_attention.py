@@ -6,7 +6,7 @@ depend on how its prompt was cut or batched. Queries are prepared in fp32 by
 ops.qkv_store, which also scatters the step's keys and values; scores,
 softmax and the per-head post-processing are fp32.
 
-Two mixers are built on it:
+Three mixers are built on it:
 
 DifferentialAttention — every head has TWO query/key maps over the same
 values. With a1, a2 the two softmax results, o = a1 - lambda * a2, then o is
@@ -24,7 +24,15 @@ consecutive positions that lies wholly outside the window, in the same
 softmax. The means are kept in the cache's pooled rows (fp32), written by
 ops.pool_cache_update when a block's last token is stored.
 
-Either mixer may read ANOTHER layer's cache rows (`owns_cache=False`) with
+GatedSigmoidAttention — no softmax: a visible key j weighs sigmoid(q . k_j *
+scale + b_h) with a learned number b_h per head, and the weights are not
+normalised over the keys. Queries and keys pass a per-head RMS norm with a
+learned weight (shared by the heads) and then a rotation by position on their
+first rot_dims dimensions (pairs i, i + rot_dims/2, YaRN frequency ramp);
+full causal mask; head h's result is multiplied by sigmoid(w_g,h . x), an
+output gate that reads the mixer's input.
+
+Any of them may read ANOTHER layer's cache rows (`owns_cache=False`) with
 its own queries. All sizes and constants are constructor arguments.
 """
 
@@ -40,6 +48,7 @@ from .. import ops
 from ..parallel.comm import get_comm
 from ..parallel.layers import MergedColumnParallelLinear, RowParallelLinear
 from .forward_meta import ForwardMeta
+from .rope import yarn_ramp_frequencies
 
 
 class _RowAttentionBase(nn.Module):
@@ -48,7 +57,7 @@ class _RowAttentionBase(nn.Module):
     def __init__(self, hidden_size: int, heads: int, kv_heads: int, dim: int,
                  value_dim: int, scale: float, norm_eps: float,
                  cache_layer_idx: int, owns_cache: bool, bias: bool,
-                 separate_values: bool):
+                 separate_values: bool, extra_sizes=(), own_proj: bool = True):
         super().__init__()
         if get_comm().tp_size != 1:
             raise NotImplementedError(
@@ -66,7 +75,13 @@ class _RowAttentionBase(nn.Module):
             sizes.append(kv_heads * self.maps * dim)
             if separate_values:
                 sizes.append(kv_heads * value_dim)
-        self.in_proj = MergedColumnParallelLinear(hidden_size, sizes, bias=bias)
+        # widths of the input projections, in order: queries, (keys, values,)
+        # then whatever the mixer adds (e.g. gate pre-activations). own_proj
+        # False: a caller merges them with other projections of the same
+        # input and hands the parts to the mixer's mix()
+        self.proj_sizes = sizes + list(extra_sizes)
+        self.in_proj = MergedColumnParallelLinear(
+            hidden_size, self.proj_sizes, bias=bias) if own_proj else None
         self.o_proj = RowParallelLinear(heads * value_dim, hidden_size)
 
     def _project(self, x: torch.Tensor):
@@ -154,3 +169,66 @@ class PooledWindowAttention(_RowAttentionBase):
             query_bounds=meta.query_bounds(),
         )
         return self.o_proj(o)
+
+
+class GatedSigmoidAttention(_RowAttentionBase):
+    maps = 1
+
+    def __init__(self, hidden_size: int, heads: int, kv_heads: int, dim: int,
+                 value_dim: int, scale: float, norm_eps: float,
+                 cache_layer_idx: int, owns_cache: bool = True,
+                 rot_dims: int = 0, rot_base: float = 10000.0,
+                 rot_scaling: Optional[dict] = None, own_proj: bool = True):
+        super().__init__(hidden_size, heads, kv_heads, dim, value_dim, scale,
+                         norm_eps, cache_layer_idx, owns_cache, False, True,
+                         extra_sizes=[heads], own_proj=own_proj)
+        if rot_dims % 2 or rot_dims > dim:
+            raise ValueError(f"cannot rotate {rot_dims} of {dim} dimensions")
+        self.rot_dims = int(rot_dims)
+        sc = rot_scaling or {}
+        self._freq, self._mult = (None, 1.0)
+        if self.rot_dims:
+            self._freq, self._mult = yarn_ramp_frequencies(
+                self.rot_dims, rot_base, float(sc.get("factor", 1.0)),
+                float(sc.get("original", 0.0)), float(sc.get("fast", 32.0)),
+                float(sc.get("slow", 1.0)))
+        self.q_norm = nn.Parameter(torch.empty(dim), requires_grad=False)
+        self.k_norm = nn.Parameter(torch.empty(dim), requires_grad=False)
+        self.score_bias = nn.Parameter(torch.empty(heads), requires_grad=False)
+        self._f32 = None
+
+    def invalidate_constants(self) -> None:
+        self._f32 = None
+
+    def _constants(self, device):
+        if self._f32 is None or self._f32[0].device != device:
+            self._f32 = (
+                self.q_norm.detach().float().contiguous().to(device),
+                self.k_norm.detach().float().contiguous().to(device),
+                self.score_bias.detach().float().contiguous().to(device),
+                self._freq.to(device) if self._freq is not None else None,
+            )
+        return self._f32
+
+    def mix(self, parts, meta: ForwardMeta, out_dtype) -> torch.Tensor:
+        """parts: the projections [q, (k, v,) gate pre-activations] of the
+        step's tokens (strided views are fine) -> [T, heads * value_dim]."""
+        q, gate = parts[0], parts[-1]
+        k, v = (parts[1], parts[2]) if self.owns_cache else (None, None)
+        wq, wk, bias, freq = self._constants(q.device)
+        cache = meta.mla_cache.layer(self.cache_layer_idx)
+        q32 = ops.qkv_store(q, k, v, meta.positions, meta.slot_mapping, cache,
+                            self.dim, self.eps, 0.0, 0, q_weight=wq,
+                            k_weight=wk, rot_freq=freq, rot_mult=self._mult,
+                            rot_dims=self.rot_dims)
+        return ops.row_attention(
+            q32, cache, None, meta.block_tables, meta.token_seq(),
+            meta.positions, self.heads, self.kv_heads, 1, self.dim, self.vdim,
+            0, 0, self.scale, 0.0, 0.0, None, 1.0, out_dtype,
+            max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
+            head_bias=bias, gate=gate,
+        )
+
+    def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        parts = self.in_proj.split_output(self.in_proj(x))
+        return self.o_proj(self.mix(parts, meta, x.dtype))

@@ -158,7 +158,7 @@ class VurizenShardModel(nn.Module):
         W = self.cfg.hidden_size
         return all(
             layer.mlp is None
-            or (W % 32 == 0 and layer.mlp.intermediate_size % 64 == 0)
+            or FusedMoE.grouped_kernel_fits(W, layer.mlp.intermediate_size)
             for layer in self.layers
         )
 

@@ -506,9 +506,12 @@ def fused_moe_forward(
     activation: str = "silu",
     limit: float = 0.0,
     bias_gate_up: Optional[torch.Tensor] = None,  # [E, 2I] bf16 (gpt-oss)
+    weight_on_input: bool = False,
 ) -> torch.Tensor:
     """Grouped-GEMM MoE (device-side routing; graph-capture safe). Returns
-    fp32 [T, H]."""
+    fp32 [T, H]. weight_on_input: the routing weight multiplies the expert's
+    input (its gate/up accumulators, before bias and activation) instead of
+    its output."""
     assert x.is_cuda
     ext = _require_ext("moe_forward")
     T, H = x.shape
@@ -524,7 +527,7 @@ def fused_moe_forward(
     ext.moe_forward(out, x.contiguous(), w_gate_up, w_down, perm.contiguous(),
                     seg.contiguous(), route_w, k, activation == "gelu", limit,
                     bias_gate_up if bias_gate_up is not None
-                    else x.new_empty(0))
+                    else x.new_empty(0), bool(weight_on_input))
     return out
 
 
@@ -646,11 +649,14 @@ apply_penalties = ref.apply_penalties
 # -- sequence mixers (extension _mix) ------------------------------------------
 from .mix import (  # noqa: E402,F401
     add_layernorm,
+    branch_rmsnorm_add,
+    clamped_glu,
     gated_rmsnorm,
     gla_recurrence,
     has_mix_extension,
     latent_kv_store,
     latent_window_attention,
+    mingru_scan,
     pool_cache_update,
     qkv_store,
     rope_rows,

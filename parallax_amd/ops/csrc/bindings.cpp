@@ -53,7 +53,8 @@ void launch_msa_paged_attention_decode(void*, const void*, const void*,
 void launch_build_moe_tiles(int*, int*, const int*, int, int, hipStream_t);
 void launch_moe_gate_up(void*, const void*, const void*, const int*,
                         const int*, const int64_t*, const int*, int, int, int,
-                        int, int, bool, float, const void*, hipStream_t);
+                        int, int, bool, float, const void*, const float*,
+                        hipStream_t);
 void launch_moe_down(void*, const void*, const void*, const float*, const int*,
                      const int*, const int64_t*, const int*, int, int, int,
                      int, int, hipStream_t);
@@ -414,7 +415,7 @@ void moe_forward(torch::Tensor out, torch::Tensor x, torch::Tensor w_gu,
                  torch::Tensor w_down, torch::Tensor perm,
                  torch::Tensor seg_offsets, torch::Tensor route_w,
                  int64_t topk, bool gelu, double limit,
-                 torch::Tensor bias_gu) {
+                 torch::Tensor bias_gu, bool weight_on_input) {
   CHECK_GPU(x);
   CHECK_CONTIG(x);
   CHECK_BF16(x);
@@ -428,8 +429,8 @@ void moe_forward(torch::Tensor out, torch::Tensor x, torch::Tensor w_gu,
   const int I = w_gu.size(1) / 2;
   const int H = w_gu.size(2);
   const int n_assign = perm.size(0);
-  TORCH_CHECK(H % 32 == 0 && I % 64 == 0,
-              "MoE dims must be multiples of 32/64 (H=", H, " I=", I, ")");
+  TORCH_CHECK(H % 32 == 0 && I % 32 == 0,
+              "MoE dims must be multiples of 32 (H=", H, " I=", I, ")");
   const int max_tiles = (n_assign + 15) / 16 + E;
   auto iopts = x.options().dtype(at::kInt);
   torch::Tensor tile_expert = torch::empty({max_tiles}, iopts);
@@ -446,9 +447,12 @@ void moe_forward(torch::Tensor out, torch::Tensor x, torch::Tensor w_gu,
                      tile_expert.data_ptr<int>(), tile_row0.data_ptr<int>(),
                      perm.data_ptr<int64_t>(), seg_offsets.data_ptr<int>(), E,
                      (int)topk, H, I, max_tiles, gelu, (float)limit,
-                     bias_gu.numel() ? bias_gu.data_ptr() : nullptr, stream);
+                     bias_gu.numel() ? bias_gu.data_ptr() : nullptr,
+                     weight_on_input ? route_w.data_ptr<float>() : nullptr,
+                     stream);
   launch_moe_down(out.data_ptr(), h_buf.data_ptr(), w_down.data_ptr(),
-                  route_w.data_ptr<float>(), tile_expert.data_ptr<int>(),
+                  weight_on_input ? nullptr : route_w.data_ptr<float>(),
+                  tile_expert.data_ptr<int>(),
                   tile_row0.data_ptr<int>(), perm.data_ptr<int64_t>(),
                   seg_offsets.data_ptr<int>(), E, (int)topk, H, I, max_tiles,
                   stream);

@@ -7,6 +7,9 @@
 //   moe_gate_up:      h = act(x[gather] @ W_gu[e]^T)   (gate/up column pairs
 //                     land in the same lane -> activation fused in-register)
 //   moe_down:         out[t] += route_w * (h @ W_down[e]^T)  (fp32 atomics)
+// With in_w the routing weight multiplies the expert's INPUT instead: the
+// gate/up accumulators are scaled by it (both projections are linear) and
+// moe_down adds the result unweighted.
 //
 // Shapes: W_gu [E, 2I, H], W_down [E, H, I] (row-major, out-major) — B operand
 // fragments read rows k-consecutive, so no transposition anywhere. Fixed
@@ -53,7 +56,8 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
     const int* __restrict__ seg_offsets,   // [E+1]
     const int E, const int topk, const int H, const int I,
     const float limit,                     // >0: gpt-oss clamped act
-    const uint16_t* __restrict__ bias_gu = nullptr) {  // [E, 2I] or null
+    const uint16_t* __restrict__ bias_gu = nullptr,  // [E, 2I] or null
+    const float* __restrict__ in_w = nullptr) {  // [T*k] sorted, or null
   const int tile = blockIdx.x;
   const int e = tile_expert[tile];
   if (e < 0) return;
@@ -67,6 +71,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
   const int l4 = lane >> 4;
 
   const int n0 = blockIdx.y * 64 + wid * 16;  // column tile within I
+  if (n0 >= I) return;  // I is a multiple of 16, not necessarily of 64
   // gate row n0+l15 of W_gu; up row I+n0+l15
   const uint16_t* wg_row = w_gu + ((size_t)e * 2 * I + (n0 + l15)) * H;
   const uint16_t* wu_row = w_gu + ((size_t)e * 2 * I + (I + n0 + l15)) * H;
@@ -107,6 +112,11 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
       if (grow >= rows_end) continue;
       const int n = n0 + l15;              // column within I
       float g = acc_g[mt][r], u = acc_u[mt][r];
+      if (in_w != nullptr) {
+        const float w = in_w[grow];
+        g *= w;
+        u *= w;
+      }
       if (bias_gu != nullptr) {
         g += bf16_bits_to_f32(bias_gu[(size_t)e * 2 * I + n]);
         u += bf16_bits_to_f32(bias_gu[(size_t)e * 2 * I + I + n]);
@@ -195,7 +205,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
       for (int r = 0; r < 4; ++r) {
         const int grow = row0 + mt * 16 + l4 * 4 + r;
         if (grow >= rows_end) continue;
-        const float w = route_w[grow];
+        const float w = route_w != nullptr ? route_w[grow] : 1.f;
         const int64_t token = perm[grow] / topk;
         atomicAdd(out + (size_t)token * H + n, acc[mt][nt][r] * w);
       }
@@ -453,18 +463,18 @@ extern "C" void launch_moe_gate_up(
     void* h_buf, const void* x, const void* w_gu, const int* tile_expert,
     const int* tile_row0, const int64_t* perm, const int* seg_offsets, int E,
     int topk, int H, int I, int max_tiles, bool gelu, float limit,
-    const void* bias_gu, hipStream_t stream) {
+    const void* bias_gu, const float* in_w, hipStream_t stream) {
   dim3 grid(max_tiles, ceil_div(I, 64), 1);
   if (gelu)
     moe_gate_up_kernel<true><<<grid, MOE_THREADS, 0, stream>>>(
         (uint16_t*)h_buf, (const uint16_t*)x, (const uint16_t*)w_gu,
         tile_expert, tile_row0, perm, seg_offsets, E, topk, H, I, limit,
-        (const uint16_t*)bias_gu);
+        (const uint16_t*)bias_gu, in_w);
   else
     moe_gate_up_kernel<false><<<grid, MOE_THREADS, 0, stream>>>(
         (uint16_t*)h_buf, (const uint16_t*)x, (const uint16_t*)w_gu,
         tile_expert, tile_row0, perm, seg_offsets, E, topk, H, I, limit,
-        (const uint16_t*)bias_gu);
+        (const uint16_t*)bias_gu, in_w);
 }
 
 extern "C" void launch_moe_down(

@@ -1,7 +1,8 @@
 """Sequence-mixer ops: layer norm over an fp32 residual stream, sliding-window
 attention over a compressed latent cache, gated linear attention; sandwich
 RMS norm with depth-weighted averaging, row-cache attention (differential /
-pooled sliding window) and xIELU.
+pooled sliding window / sigmoid-weighted with an output gate) and xIELU;
+post-norm residual step, minGRU scan and the clamped gated linear unit.
 
 GPU tensors go to the hand-written gfx950 kernels of the in-tree extension
 ``parallax_amd.ops._mix`` (bf16 or float32 activations; scores, norms, decays
@@ -173,21 +174,32 @@ def sandwich_rmsnorm(x, y, w_branch, hist, n_hist, dwa, w_next, eps, offset,
 
 
 def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
-              temp_coef, temp_every):
-    """Queries to fp32 (optionally RMS-normed per seg_dim-wide segment and
-    multiplied by a position-dependent temperature); keys (normed alike) and
-    values scattered as one row [keys | values] per token into the paged
-    cache. v None: values = the keys before the norm. k None: no store."""
+              temp_coef, temp_every, q_weight=None, k_weight=None,
+              rot_freq=None, rot_mult=1.0, rot_dims=0):
+    """Queries to fp32 (optionally RMS-normed per seg_dim-wide segment, with
+    a weight [seg_dim] shared by the segments, rotated by position on each
+    segment's first rot_dims dimensions (pairs i, i + rot_dims/2; angles pos *
+    rot_freq[i] in fp32 inside the kernel) and multiplied by a
+    position-dependent temperature); keys (normed, weighted and rotated
+    alike) and values scattered as one row [keys | values] per token into the
+    paged cache. v None: values = the keys before the norm. k None: no
+    store."""
     if not q.is_cuda:
         return ref.qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim,
-                             norm_eps, temp_coef, temp_every)
+                             norm_eps, temp_coef, temp_every, q_weight,
+                             k_weight, rot_freq, rot_mult, rot_dims)
     out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     e = _empty(q)
+    ef = _empty(q, torch.float32)
     _mix_ext().qkv_store(
         out, q, k if k is not None else e, v if v is not None else e,
         positions, slot_mapping, cache, int(seg_dim),
         float(norm_eps) if norm_eps is not None else -1.0,
         float(temp_coef), int(temp_every),
+        q_weight if q_weight is not None else ef,
+        k_weight if k_weight is not None else ef,
+        rot_freq if rot_freq is not None else ef, float(rot_mult),
+        int(rot_dims) if rot_freq is not None else 0,
     )
     return out
 
@@ -209,12 +221,15 @@ def pool_cache_update(cache, pool, block_tables, token_seq, positions,
 def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0,
-                  query_bounds=None):
-    """Softmax attention of fp32 queries over paged cache rows [keys |
-    values] with grouped heads: full causal (window 0) or a sliding window
-    with pooled blocks beyond it, optional tanh soft cap, one or two score
-    maps per head (two combine as a1 - lam * a2), optional RMS norm of each
-    head's result. max_seq_len: the longest context of the batch as the host
+                  query_bounds=None, head_bias=None, gate=None):
+    """Attention of fp32 queries over paged cache rows [keys | values] with
+    grouped heads: full causal (window 0) or a sliding window with pooled
+    blocks beyond it, optional tanh soft cap, one or two score maps per head
+    (two combine as a1 - lam * a2), optional RMS norm of each head's result.
+    Key weights: softmax, or, with head_bias [heads] fp32, sigmoid(score +
+    head_bias[h]) without normalisation over the keys (one map only). gate
+    [T, heads] (fp32 pre-activations): head h's result is multiplied by
+    sigmoid(gate[t, h]). max_seq_len: the longest context of the batch as the host
     knows it (0 = the block tables' capacity); it only sizes the split of
     long key ranges over workgroups. query_bounds [B+1] int32 (prompt portions:
     tokens of sequence b are query_bounds[b] .. query_bounds[b+1], at
@@ -224,8 +239,11 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         return ref.row_attention(q, cache, pool, block_tables, token_seq,
                                  positions, heads, kv_heads, maps, dim, vdim,
                                  window, pool_tokens, scale, softcap, lam,
-                                 norm_eps, out_mult, out_dtype)
+                                 norm_eps, out_mult, out_dtype, head_bias, gate)
+    if head_bias is not None and maps != 1:
+        raise ValueError("sigmoid key weights take one score map per head")
     out = torch.empty(q.shape[0], heads * vdim, dtype=out_dtype, device=q.device)
+    ef = torch.empty(0, dtype=torch.float32, device=q.device)
     _mix_ext().row_attention(
         out, q, cache,
         pool if pool is not None else torch.empty(0, dtype=torch.float32,
@@ -238,6 +256,8 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         int(max_seq_len) or block_tables.shape[1] * cache.shape[1],
         query_bounds if query_bounds is not None and token_seq is not None
         else _empty(positions),
+        head_bias if head_bias is not None else ef,
+        gate if gate is not None else ef,
     )
     return out
 
@@ -249,4 +269,63 @@ def xielu(x, a_pos, a_neg):
         return ref.xielu(x, a_pos, a_neg)
     out = torch.empty_like(x)
     _mix_ext().xielu(out, x, float(a_pos), float(a_neg))
+    return out
+
+
+# -- post-norm residual stream, minGRU, clamped gated linear unit ----------------
+
+
+def branch_rmsnorm_add(x, y1, y2, a, b, weight, eps, out_dtype, keep_stream=True):
+    """One step of a residual stream that norms a sublayer's OUTPUT, in one
+    kernel: y = a * y1 (+ b * y2), x <- x + y / sqrt(mean(y^2) + eps) * weight
+    (x None: a new stream that starts as the normed y), everything fp32; x
+    [T, W] fp32 is updated in place. y1 / y2 have the activation dtype or fp32.
+    Returns (x, x rounded to out_dtype); keep_stream False returns (None, the
+    rounded sum) and leaves x as it was."""
+    if not y1.is_cuda:
+        return ref.branch_rmsnorm_add(x, y1, y2, a, b, weight, eps, out_dtype,
+                                      keep_stream)
+    ext = _mix_ext()
+    T, W = y1.shape
+    out = torch.empty(T, W, dtype=out_dtype, device=y1.device)
+    x_out = x
+    if keep_stream and x is None:
+        x_out = torch.empty(T, W, dtype=torch.float32, device=y1.device)
+    ef = _empty(y1, torch.float32)
+    ext.branch_rmsnorm_add(
+        x if x is not None else ef, x_out if keep_stream else ef, y1,
+        y2 if y2 is not None else _empty(y1), float(a), float(b), weight,
+        float(eps), out,
+    )
+    return (x_out if keep_stream else None), out
+
+
+def mingru_scan(zug, z_bias, u_bias, state, slots, cu, positions, out_dtype):
+    """minGRU over packed sequences: zug [T, 3 * width] (any row stride) holds
+    the pre-activations of update gate, candidate and output gate;
+    S_t = (1 - z) S_(t-1) + z c per channel with z = sigmoid(z_pre + z_bias),
+    c = u + 1/2 for u >= 0, sigmoid(u) otherwise, u = u_pre + u_bias. The fp32
+    state [slots, width] is read (or started from zero at position 0) and
+    written back. cu [B+1] int32 token bounds (None: one token each). Returns
+    S_t * silu(g_pre) as [T, width] of out_dtype."""
+    if not zug.is_cuda:
+        return ref.mingru_scan(zug, z_bias, u_bias, state, slots, cu,
+                               positions, out_dtype)
+    width = state.shape[1]
+    out = torch.empty(zug.shape[0], width, dtype=out_dtype, device=zug.device)
+    _mix_ext().mingru_scan(
+        out, zug, z_bias, u_bias, state, slots,
+        cu if cu is not None else _empty(positions), positions,
+    )
+    return out
+
+
+def clamped_glu(gate_up, limit, alpha=1.702):
+    """[gate | up] -> min(gate, limit) * sigmoid(alpha * min(gate, limit)) *
+    (clamp(up, -limit, limit) + 1), fp32 inside, result in the input dtype."""
+    if not gate_up.is_cuda:
+        return ref.clamped_glu(gate_up, limit, alpha)
+    out = torch.empty(gate_up.shape[0], gate_up.shape[1] // 2,
+                      dtype=gate_up.dtype, device=gate_up.device)
+    _mix_ext().clamped_glu(out, gate_up, float(limit), float(alpha))
     return out

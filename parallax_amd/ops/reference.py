@@ -698,17 +698,32 @@ def _segment_rms(x, seg, eps):
     return (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(T, -1)
 
 
+def _segment_rotate(x, seg, positions, freq, mult, rot_dims):
+    T = x.shape[0]
+    return _rotate_rows(x.view(T, -1, seg), positions, freq, mult,
+                        rot_dims).reshape(T, -1)
+
+
 def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
-              temp_coef, temp_every):
+              temp_coef, temp_every, q_weight=None, k_weight=None,
+              rot_freq=None, rot_mult=1.0, rot_dims=0):
     """Queries to fp32 (each seg_dim-wide segment divided by its RMS when
-    norm_eps is given; multiplied by 1 + temp_coef * ln(floor((pos + 1) /
-    temp_every) + 1) when temp_every > 0), keys (segments normed alike) and
-    values into one cache row [keys | values] per token. v None: the values
-    are the keys as they came in, before the norm. k None: nothing is stored
-    (the layer reads another layer's rows). Slot -1 skips the token."""
+    norm_eps is given, times q_weight [seg_dim] when given; then its first
+    rot_dims dimensions rotated by position, dimension i paired with i +
+    rot_dims / 2 at angle pos * rot_freq[i], cos and sin times rot_mult, when
+    rot_freq is given; multiplied by 1 + temp_coef * ln(floor((pos + 1) /
+    temp_every) + 1) when temp_every > 0), keys (segments normed, weighted by
+    k_weight and rotated alike) and values into one cache row [keys | values]
+    per token. v None: the values are the keys as they came in, before the
+    norm. k None: nothing is stored (the layer reads another layer's rows).
+    Slot -1 skips the token."""
     qf = q.float()
     if norm_eps is not None:
         qf = _segment_rms(qf, seg_dim, norm_eps)
+    if q_weight is not None:
+        qf = (qf.view(qf.shape[0], -1, seg_dim) * q_weight.float()).reshape(qf.shape)
+    if rot_freq is not None:
+        qf = _segment_rotate(qf, seg_dim, positions, rot_freq, rot_mult, rot_dims)
     if temp_every > 0:
         p = positions.float()
         temp = 1.0 + temp_coef * torch.log(torch.floor((p + 1.0) / temp_every) + 1.0)
@@ -718,6 +733,10 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
         vals = kf if v is None else v.float()
         if norm_eps is not None:
             kf = _segment_rms(kf, seg_dim, norm_eps)
+        if k_weight is not None:
+            kf = (kf.view(kf.shape[0], -1, seg_dim) * k_weight.float()).reshape(kf.shape)
+        if rot_freq is not None:
+            kf = _segment_rotate(kf, seg_dim, positions, rot_freq, rot_mult, rot_dims)
         entry = torch.cat([kf, vals], dim=-1).to(cache.dtype)
         keep = slot_mapping >= 0
         flat = cache.view(-1, cache.shape[-1])
@@ -752,8 +771,9 @@ def pool_cache_update(cache, pool, block_tables, token_seq, positions,
 
 def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
-                  softcap, lam, norm_eps, out_mult, out_dtype):
-    """Softmax attention over cache rows [keys (kv_heads x maps x dim) |
+                  softcap, lam, norm_eps, out_mult, out_dtype, head_bias=None,
+                  gate=None):
+    """Attention over cache rows [keys (kv_heads x maps x dim) |
     values (kv_heads x vdim)]. q [T, heads * maps * dim] fp32. window 0: every
     key up to the token's position; window > 0: keys j with 0 <= pos - j <
     window plus, when pool_tokens > 0, the pooled row of every block of
@@ -761,6 +781,9 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
     softmax. softcap > 0: s <- softcap * tanh(s / softcap). maps == 2: the
     two maps' results (same values) combine as a1 - lam * a2. norm_eps given:
     the head's result is divided by its RMS and multiplied by out_mult.
+    head_bias [heads] given: no softmax; a visible key weighs sigmoid(s +
+    head_bias[h]) and the weights are not normalised over the keys. gate
+    [T, heads] given: head h's result is multiplied by sigmoid(gate[t, h]).
     Returns [T, heads * vdim] in out_dtype."""
     T = q.shape[0]
     bs = cache.shape[1]
@@ -787,10 +810,16 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         s = torch.einsum("grmd,ngmd->grmn", qv[t], k) * scale
         if softcap > 0:
             s = softcap * torch.tanh(s / softcap)
-        a = torch.einsum("grmn,ngv->grmv", torch.softmax(s, dim=-1), v)
+        if head_bias is not None:
+            wts = torch.sigmoid(s + head_bias.float().view(G, rep, 1, 1))
+        else:
+            wts = torch.softmax(s, dim=-1)
+        a = torch.einsum("grmn,ngv->grmv", wts, v)
         o = a[:, :, 0] - lam * a[:, :, 1] if M == 2 else a[:, :, 0]
         if norm_eps is not None:
             o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + norm_eps) * out_mult
+        if gate is not None:
+            o = o * torch.sigmoid(gate[t].float()).view(G, rep, 1)
         out[t] = o.reshape(H, vdim)
     return out.view(T, H * vdim).to(out_dtype)
 
@@ -802,3 +831,70 @@ def xielu(x, a_pos, a_neg):
     out = torch.where(z > 0, a_pos * z * z + 0.5 * z,
                       (0.5 + a_neg) * (torch.expm1(neg) - neg) + 0.5 * z)
     return out.to(x.dtype)
+
+
+# -- post-norm residual stream, minGRU, clamped gated linear unit ----------------
+
+
+def branch_rmsnorm_add(x, y1, y2, a, b, weight, eps, out_dtype, keep_stream=True):
+    """One step of a residual stream that norms a sublayer's OUTPUT:
+      y = a * y1 (+ b * y2),  n = y / sqrt(mean(y^2) + eps) * weight,
+      x <- x + n   (x None: x = n)
+    all in fp32; x [T, W] fp32 is updated in place. Returns (x, x in
+    out_dtype); keep_stream False: (None, the sum in out_dtype) and x is
+    left as it was."""
+    y = a * y1.float()
+    if y2 is not None:
+        y = y + b * y2.float()
+    n = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float()
+    if x is not None:
+        n = n + x
+    if not keep_stream:
+        return None, n.to(out_dtype)
+    if x is None:
+        x = n.contiguous()
+    else:
+        x.copy_(n)
+    return x, x.to(out_dtype)
+
+
+def mingru_scan(zug, z_bias, u_bias, state, slots, cu, positions, out_dtype):
+    """minGRU over packed sequences. zug [T, 3 * width]: pre-activations of
+    the update gate z, the candidate u and the output gate g of every token.
+      z = sigmoid(z_pre + z_bias),  c = u + 1/2 (u >= 0) | sigmoid(u) (u < 0)
+      with u = u_pre + u_bias,      S_t = (1 - z) S_(t-1) + z c   per channel,
+    fp32 throughout; the state [slots, width] fp32 is read (or started from
+    zero when the portion begins at position 0) and written back. cu [B+1]
+    int32 token bounds (None: one token each). Returns S_t * silu(g_pre) as
+    [T, width] of out_dtype."""
+    T = zug.shape[0]
+    width = state.shape[1]
+    f = zug.float()
+    z = torch.sigmoid(f[:, :width] + z_bias.float())
+    u = f[:, width : 2 * width] + u_bias.float()
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = f[:, 2 * width :]
+    g = g * torch.sigmoid(g)
+    out = torch.empty(T, width, dtype=torch.float32)
+    bounds = cu.tolist() if cu is not None else list(range(T + 1))
+    pos = positions.tolist()
+    for b, slot in enumerate(slots.tolist()):
+        t0, t1 = bounds[b], bounds[b + 1]
+        if t0 >= t1:
+            continue
+        S = torch.zeros(width) if pos[t0] == 0 else state[slot].clone()
+        for t in range(t0, t1):
+            S = (1.0 - z[t]) * S + z[t] * cand[t]
+            out[t] = S * g[t]
+        state[slot] = S
+    return out.to(out_dtype)
+
+
+def clamped_glu(gate_up, limit, alpha=1.702):
+    """gate_up [T, 2 I] = [gate | up]: g = min(gate, limit), u = clamp(up,
+    -limit, limit); g * sigmoid(alpha * g) * (u + 1) -> [T, I] (fp32 inside)."""
+    I = gate_up.shape[-1] // 2
+    f = gate_up.float()
+    g = f[..., :I].clamp(max=limit)
+    u = f[..., I:].clamp(min=-limit, max=limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate_up.dtype)
