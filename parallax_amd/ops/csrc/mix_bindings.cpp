@@ -39,7 +39,8 @@ void launch_sandwich_rmsnorm(float*, const void*, int64_t, int, const void*,
 void launch_xielu(void*, const void*, int64_t, float, float, int, hipStream_t);
 void launch_qkv_store(float*, const void*, int64_t, const void*, int64_t,
                       const void*, int64_t, const int*, const int64_t*, void*,
-                      int, int, int, int, float, float, int, int, int,
+                      int, int, int, int, float, float, int, const float*,
+                      const float*, const float*, float, int, int, int,
                       hipStream_t);
 void launch_pool_cache_update(const void*, float*, const int*, int, const int*,
                               const int*, const int64_t*, int, int, int, int,
@@ -49,13 +50,22 @@ int row_attention_prefill_supported(int, int);
 void launch_row_attention_prefill(void*, const float*, const void*, const float*,
                                   const int*, int, const int*, int, const int*,
                                   int, int, int, int, int, int, int, int, int,
-                                  int, float, float, float, float, float, int,
+                                  int, float, float, float, float, float,
+                                  const float*, const void*, int64_t, int,
                                   hipStream_t);
 void launch_row_attention(void*, float*, const float*, const void*,
                           const float*, const int*, int, const int*, const int*,
                           int, int, int, int, int, int, int, int, int, int,
-                          float, float, float, float, float, int, int,
-                          hipStream_t);
+                          float, float, float, float, float, int, const float*,
+                          const void*, int64_t, int, hipStream_t);
+void launch_branch_rmsnorm_add(const float*, float*, const void*, int64_t, int,
+                               const void*, int64_t, float, float, const void*,
+                               float, void*, int, int, int, hipStream_t);
+void launch_clamped_glu(void*, const void*, int64_t, int, int, float, float,
+                        int, hipStream_t);
+void launch_mingru_scan(void*, const void*, int64_t, const float*, const float*,
+                        float*, const int64_t*, const int*, const int*, int,
+                        int, int, hipStream_t);
 }
 
 static hipStream_t cur_stream() {
@@ -360,8 +370,27 @@ void xielu(torch::Tensor out, torch::Tensor x, double a_pos, double a_neg) {
 void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                torch::Tensor v, torch::Tensor positions, torch::Tensor slots,
                torch::Tensor cache, int64_t seg, double eps, double temp_coef,
-               int64_t temp_every) {
+               int64_t temp_every, torch::Tensor q_weight,
+               torch::Tensor k_weight, torch::Tensor rot_freq, double rot_mult,
+               int64_t rot_dims) {
   const int kind = kind_of(q, "q");
+  const bool has_qw = q_weight.numel() > 0, has_kw = k_weight.numel() > 0;
+  const bool has_rot = rot_freq.numel() > 0 && rot_dims > 0;
+  if (has_qw || has_kw || has_rot)
+    TORCH_CHECK(seg > 0 && q.size(1) % seg == 0, "query width / segment");
+  if (has_qw) {
+    CHECK_F32C(q_weight);
+    TORCH_CHECK(q_weight.numel() == seg, "query norm weight width");
+  }
+  if (has_kw) {
+    CHECK_F32C(k_weight);
+    TORCH_CHECK(k_weight.numel() == seg, "key norm weight width");
+  }
+  if (has_rot) {
+    CHECK_F32C(rot_freq);
+    TORCH_CHECK(rot_dims % 2 == 0 && rot_dims <= seg &&
+                rot_freq.numel() == rot_dims / 2, "rotated dimensions");
+  }
   CHECK_F32C(q_out);
   TORCH_CHECK(q.dim() == 2 && q.stride(1) == 1 && q_out.dim() == 2);
   const int T = q.size(0), wq = q.size(1);
@@ -376,7 +405,8 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
     TORCH_CHECK(k.is_cuda() && k.scalar_type() == q.scalar_type() &&
                 k.dim() == 2 && k.size(0) == T && k.stride(1) == 1);
     wk = k.size(1);
-    if (eps >= 0) TORCH_CHECK(wk % seg == 0, "key width / segment");
+    if (eps >= 0 || has_kw || has_rot)
+      TORCH_CHECK(wk % seg == 0, "key width / segment");
     if (has_v) {
       TORCH_CHECK(v.is_cuda() && v.scalar_type() == q.scalar_type() &&
                   v.dim() == 2 && v.size(0) == T && v.stride(1) == 1);
@@ -396,7 +426,11 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                    positions.data_ptr<int>(),
                    has_k ? slots.data_ptr<int64_t>() : nullptr,
                    has_k ? cache.data_ptr() : nullptr, wq, wk, wv, (int)seg,
-                   (float)eps, (float)temp_coef, (int)temp_every, T, kind,
+                   (float)eps, (float)temp_coef, (int)temp_every,
+                   has_qw ? q_weight.data_ptr<float>() : nullptr,
+                   has_kw ? k_weight.data_ptr<float>() : nullptr,
+                   has_rot ? rot_freq.data_ptr<float>() : nullptr,
+                   (float)rot_mult, has_rot ? (int)rot_dims : 0, T, kind,
                    cur_stream());
 }
 
@@ -438,9 +472,24 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
                    int64_t G, int64_t M, int64_t d, int64_t dv, int64_t window,
                    int64_t P, double scale, double softcap, double lam,
                    double norm_eps, double out_mult, int64_t max_keys,
-                   torch::Tensor query_bounds) {
+                   torch::Tensor query_bounds, torch::Tensor head_bias,
+                   torch::Tensor gate) {
   const int kind = kind_of(cache, "cache");
   CHECK_F32C(q);
+  // head_bias [H] fp32: sigmoid(score + head_bias[h]) weights, not normalised;
+  // gate [T, H] (cache type, row stride free): result times sigmoid(gate)
+  const bool has_bias = head_bias.numel() > 0, has_gate = gate.numel() > 0;
+  if (has_bias) {
+    CHECK_F32C(head_bias);
+    TORCH_CHECK(head_bias.numel() == H && M == 1, "head bias");
+  }
+  if (has_gate)
+    TORCH_CHECK(gate.is_cuda() && gate.scalar_type() == cache.scalar_type() &&
+                gate.dim() == 2 && gate.size(0) == q.size(0) &&
+                gate.size(1) == H && gate.stride(1) == 1, "gate");
+  const float* bias_p = has_bias ? head_bias.data_ptr<float>() : nullptr;
+  const void* gate_p = has_gate ? gate.data_ptr() : nullptr;
+  const int64_t gate_stride = has_gate ? gate.stride(0) : 0;
   TORCH_CHECK(q.dim() == 2 && cache.dim() == 3 && cache.is_contiguous());
   const int T = q.size(0);
   TORCH_CHECK(H >= 1 && G >= 1 && H % G == 0 && (M == 1 || M == 2) && d >= 1 &&
@@ -488,7 +537,7 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
         (T + 31) / 32 + B, (int)H, (int)G, (int)M, (int)d, (int)dv,
         (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
         (float)scale, (float)softcap, (float)lam, (float)norm_eps,
-        (float)out_mult, kind, cur_stream());
+        (float)out_mult, bias_p, gate_p, gate_stride, kind, cur_stream());
     return;
   }
   // shares of the key list per token: enough workgroups to fill the chip
@@ -519,7 +568,90 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
       positions.data_ptr<int>(), T, (int)H, (int)G, (int)M, (int)d, (int)dv,
       (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
       (float)scale, (float)softcap, (float)lam, (float)norm_eps,
-      (float)out_mult, splits, kind, cur_stream());
+      (float)out_mult, splits, bias_p, gate_p, gate_stride, kind, cur_stream());
+}
+
+// x_in [T, W] fp32 or empty; x_out [T, W] fp32 or empty (may be x_in); y1
+// [T, W] activation type or fp32, y2 [T, W] activation type or empty (row
+// strides free); weight [W] and out [T, W] of the activation type
+void branch_rmsnorm_add(torch::Tensor x_in, torch::Tensor x_out,
+                        torch::Tensor y1, torch::Tensor y2, double a, double b,
+                        torch::Tensor weight, double eps, torch::Tensor out) {
+  const int kind = kind_of(out, "out");
+  const int y1_kind = kind_of(y1, "y1");
+  TORCH_CHECK(y1.dim() == 2 && y1.stride(1) == 1 && out.dim() == 2 &&
+              out.is_contiguous());
+  const int T = y1.size(0), W = y1.size(1);
+  TORCH_CHECK(out.size(0) == T && out.size(1) == W);
+  TORCH_CHECK(kind == 0 || y1_kind == 1, "fp32 stacks take fp32 branches");
+  TORCH_CHECK(weight.is_cuda() && weight.scalar_type() == out.scalar_type() &&
+              weight.is_contiguous() && weight.numel() == W, "norm weight");
+  const bool has_x = x_in.numel() > 0, has_o = x_out.numel() > 0;
+  if (has_x) {
+    CHECK_F32C(x_in);
+    TORCH_CHECK(x_in.dim() == 2 && x_in.size(0) == T && x_in.size(1) == W);
+  }
+  if (has_o) {
+    CHECK_F32C(x_out);
+    TORCH_CHECK(x_out.dim() == 2 && x_out.size(0) == T && x_out.size(1) == W);
+  }
+  const bool has_y2 = y2.numel() > 0;
+  if (has_y2)
+    TORCH_CHECK(y2.is_cuda() && y2.scalar_type() == out.scalar_type() &&
+                y2.dim() == 2 && y2.size(0) == T && y2.size(1) == W &&
+                y2.stride(1) == 1, "second branch");
+  launch_branch_rmsnorm_add(
+      has_x ? x_in.data_ptr<float>() : nullptr,
+      has_o ? x_out.data_ptr<float>() : nullptr, y1.data_ptr(), y1.stride(0),
+      y1_kind, has_y2 ? y2.data_ptr() : nullptr, has_y2 ? y2.stride(0) : 0,
+      (float)a, (float)b, weight.data_ptr(), (float)eps, out.data_ptr(), T, W,
+      kind, cur_stream());
+}
+
+// x [T, 2 I] (row stride free) -> out [T, I]
+void clamped_glu(torch::Tensor out, torch::Tensor x, double limit, double alpha) {
+  const int kind = kind_of(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && x.size(1) % 2 == 0);
+  const int T = x.size(0), I = x.size(1) / 2;
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == x.scalar_type() &&
+              out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == I);
+  launch_clamped_glu(out.data_ptr(), x.data_ptr(), x.stride(0), T, I,
+                     (float)limit, (float)alpha, kind, cur_stream());
+}
+
+// zug [T, 3 width] (row stride free); state [slots, width] fp32; slots [B]
+// int64; cu [B + 1] int32 or empty (one token per sequence); out [T, width]
+void mingru_scan(torch::Tensor out, torch::Tensor zug, torch::Tensor z_bias,
+                 torch::Tensor u_bias, torch::Tensor state, torch::Tensor slots,
+                 torch::Tensor cu, torch::Tensor positions) {
+  const int kind = kind_of(zug, "zug");
+  CHECK_F32C(z_bias);
+  CHECK_F32C(u_bias);
+  CHECK_F32C(state);
+  CHECK_I64(slots);
+  CHECK_I32(positions);
+  TORCH_CHECK(state.dim() == 2 && zug.dim() == 2 && zug.stride(1) == 1);
+  const int T = zug.size(0), width = state.size(1);
+  TORCH_CHECK(zug.size(1) == 3 * width && z_bias.numel() == width &&
+              u_bias.numel() == width, "minGRU widths");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == zug.scalar_type() &&
+              out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == width);
+  TORCH_CHECK(positions.numel() == T);
+  const int B = slots.numel();
+  const bool has_cu = cu.numel() > 0;
+  if (has_cu) {
+    CHECK_I32(cu);
+    TORCH_CHECK(cu.numel() == B + 1);
+  } else {
+    TORCH_CHECK(B == T, "one token per sequence without token bounds");
+  }
+  launch_mingru_scan(out.data_ptr(), zug.data_ptr(), zug.stride(0),
+                     z_bias.data_ptr<float>(), u_bias.data_ptr<float>(),
+                     state.data_ptr<float>(), slots.data_ptr<int64_t>(),
+                     has_cu ? cu.data_ptr<int>() : nullptr,
+                     positions.data_ptr<int>(), B, width, kind, cur_stream());
 }
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -534,4 +666,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("qkv_store", &qkv_store);
   m.def("pool_cache_update", &pool_cache_update);
   m.def("row_attention", &row_attention);
+  m.def("branch_rmsnorm_add", &branch_rmsnorm_add);
+  m.def("clamped_glu", &clamped_glu);
+  m.def("mingru_scan", &mingru_scan);
 }

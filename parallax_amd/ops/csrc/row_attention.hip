@@ -1,4 +1,6 @@
-// Grouped-head softmax attention over a row-per-token paged cache.
+// Grouped-head attention over a row-per-token paged cache: softmax weights,
+// or sigmoid(score + per-head bias) weights that are not normalised over the
+// keys; optionally a per-head sigmoid gate on the result.
 //
 // A cache row holds, for one token, the keys of all kv heads and then the
 // values of all kv heads: [G x M x d | G x dv], M = score maps per head (1, or
@@ -7,11 +9,13 @@
 // accumulation and the per-head post-processing are fp32; only the cache rows
 // and the result have the activation type.
 //
-//   qkv_store         : queries -> fp32 (optional per-segment RMS norm, optional
-//                       position-dependent temperature); keys (normed alike)
-//                       and values scattered into the token's cache row. With
-//                       no value tensor the values are the keys BEFORE the
-//                       norm.
+//   qkv_store         : queries -> fp32 (optional per-segment RMS norm with an
+//                       optional weight, optional rotation by position of the
+//                       segment's first dimensions, optional
+//                       position-dependent temperature); keys (normed,
+//                       weighted and rotated alike) and values scattered into
+//                       the token's cache row. With no value tensor the
+//                       values are the keys BEFORE the norm.
 //   pool_cache_update : a token that completes a block of P positions writes
 //                       the fp32 mean of the block's P cache rows to the
 //                       sequence's pooled rows.
@@ -30,29 +34,68 @@
 //                       workgroups, sized from host-known numbers only, and
 //                       row_attention_reduce joins the partial results.
 //   epilogue          : o = a1 - lam * a2 (M = 2) or a1; optional division by
-//                       the RMS over the value width, times out_mult.
+//                       the RMS over the value width, times out_mult;
+//                       optional sigmoid(gate[t, h]) multiplier.
+//   sigmoid weights   : with head_bias a visible key weighs sigmoid(score +
+//                       head_bias[h]); the running maximum is pinned at 0
+//                       and the denominator at 1, so partial results of
+//                       waves and key shares simply add up.
 #include "seq_common.h"
 
 #define RA_WAVES 4
 
 // ---- qkv_store -------------------------------------------------------------
 
+// What a segment passes after its norm: a weight per dimension (shared by the
+// segments) and a rotation of its first rot_dims dimensions by the token's
+// position, dimension i paired with i + rot_dims / 2 at angle pos * freq[i]
+// (fp32), cos and sin times rot_mult.
+struct RaSegOps {
+  const float* w;      // [seg] or null
+  const float* freq;   // [rot_dims / 2] or null
+  float rot_mult;
+  int rot_dims;
+  float pos;
+};
+
 // n elements in segments of `seg`; NORM: every segment divided by its RMS
 // (wave per segment), then times mult.
 template <typename TI, typename TO, bool NORM>
 DEVINL void ra_segments(const TI* __restrict__ src, TO* __restrict__ dst, int n,
-                        int seg, float eps, float mult) {
-  if (NORM) {
+                        int seg, float eps, float mult, const RaSegOps& so) {
+  if (NORM || so.w != nullptr || so.freq != nullptr) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = so.freq ? so.rot_dims / 2 : 0;
     for (int s0 = wave * seg; s0 < n; s0 += RA_WAVES * seg) {
-      float ss = 0.f;
-      for (int i = lane; i < seg; i += 64) {
-        const float t = ldf(src + s0 + i);
-        ss += t * t;
+      float r = mult;
+      if (NORM) {
+        float ss = 0.f;
+        for (int i = lane; i < seg; i += 64) {
+          const float t = ldf(src + s0 + i);
+          ss += t * t;
+        }
+        ss = wave_reduce_sum(ss);
+        r = mult / sqrtf(ss / (float)seg + eps);
       }
-      ss = wave_reduce_sum(ss);
-      const float r = mult / sqrtf(ss / (float)seg + eps);
-      for (int i = lane; i < seg; i += 64) stf(dst + s0 + i, ldf(src + s0 + i) * r);
+      for (int i = lane; i < seg; i += 64) {
+        if (i < half) {
+          float u = ldf(src + s0 + i) * r, v = ldf(src + s0 + i + half) * r;
+          if (so.w) {
+            u *= so.w[i];
+            v *= so.w[i + half];
+          }
+          float sn, cs;
+          sincosf(so.pos * so.freq[i], &sn, &cs);
+          sn *= so.rot_mult;
+          cs *= so.rot_mult;
+          stf(dst + s0 + i, u * cs - v * sn);
+          stf(dst + s0 + i + half, v * cs + u * sn);
+        } else if (i >= 2 * half) {
+          float t = ldf(src + s0 + i) * r;
+          if (so.w) t *= so.w[i];
+          stf(dst + s0 + i, t);
+        }
+      }
     }
   } else {
     for (int i = threadIdx.x; i < n; i += 64 * RA_WAVES)
@@ -66,17 +109,22 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
     const T* __restrict__ k, int64_t k_stride, const T* __restrict__ v,
     int64_t v_stride, const int* __restrict__ positions,
     const int64_t* __restrict__ slots, T* __restrict__ cache, int wq, int wk,
-    int wv, int seg, float eps, float temp_coef, int temp_every) {
+    int wv, int seg, float eps, float temp_coef, int temp_every,
+    const float* __restrict__ q_weight, const float* __restrict__ k_weight,
+    const float* __restrict__ rot_freq, float rot_mult, int rot_dims) {
   const int64_t t = blockIdx.x;
   float temp = 1.0f;
   if (temp_every > 0)
     temp = 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f);
-  ra_segments<T, float, NORM>(q + t * q_stride, q_out + t * wq, wq, seg, eps, temp);
+  RaSegOps so{q_weight, rot_freq, rot_mult, rot_dims, (float)positions[t]};
+  ra_segments<T, float, NORM>(q + t * q_stride, q_out + t * wq, wq, seg, eps,
+                              temp, so);
   if (k == nullptr) return;
   const int64_t slot = slots[t];
   if (slot < 0) return;  // pad row of a captured graph
   T* row = cache + slot * (int64_t)(wk + wv);
-  ra_segments<T, T, NORM>(k + t * k_stride, row, wk, seg, eps, 1.0f);
+  so.w = k_weight;
+  ra_segments<T, T, NORM>(k + t * k_stride, row, wk, seg, eps, 1.0f, so);
   const T* vals = v ? v + t * v_stride : k + t * k_stride;
   for (int i = threadIdx.x; i < wv; i += 64 * RA_WAVES) row[wk + i] = vals[i];
 }
@@ -86,13 +134,16 @@ extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
                                  int64_t v_stride, const int* positions,
                                  const int64_t* slots, void* cache, int wq,
                                  int wk, int wv, int seg, float eps,
-                                 float temp_coef, int temp_every, int T_,
-                                 int kind, hipStream_t stream) {
+                                 float temp_coef, int temp_every,
+                                 const float* q_weight, const float* k_weight,
+                                 const float* rot_freq, float rot_mult,
+                                 int rot_dims, int T_, int kind,
+                                 hipStream_t stream) {
   if (T_ == 0) return;
 #define QS_ARGS(TT)                                                          \
   q_out, (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v,       \
       v_stride, positions, slots, (TT*)cache, wq, wk, wv, seg, eps,          \
-      temp_coef, temp_every
+      temp_coef, temp_every, q_weight, k_weight, rot_freq, rot_mult, rot_dims
   const bool norm = eps >= 0.f;
   if (kind == 0) {
     if (norm)
@@ -246,7 +297,7 @@ DEVINL void ra_dot(const TK* __restrict__ key, const float* __restrict__ qs,
 template <typename T, int M>
 DEVINL void ra_epilogue(T* __restrict__ dst, const float* __restrict__ acc,
                         int acc_stride, const float* l, int dv, float lam,
-                        float norm_eps, float out_mult) {
+                        float norm_eps, float out_mult, float post) {
   const int lane = threadIdx.x & 63;
   const float i0 = 1.0f / l[0];
   const float i1 = M == 2 ? lam / l[1] : 0.f;
@@ -263,16 +314,25 @@ DEVINL void ra_epilogue(T* __restrict__ dst, const float* __restrict__ acc,
     o[c] = v;
     ss += v * v;
   }
-  float r = 1.0f;
+  float r = post;
   if (norm_eps >= 0.f) {
     ss = wave_reduce_sum(ss);
-    r = out_mult / sqrtf(ss / (float)dv + norm_eps);
+    r = post * out_mult / sqrtf(ss / (float)dv + norm_eps);
   }
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int f = lane + 64 * c;
     if (f < dv) stf(dst + f, o[c] * r);
   }
+}
+
+DEVINL float ra_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// sigmoid(gate[t, h]) or 1
+template <typename T>
+DEVINL float ra_gate(const T* __restrict__ gate, int64_t gate_stride, int64_t t,
+                     int h) {
+  return gate ? ra_sigmoid(ldf(gate + t * gate_stride + h)) : 1.0f;
 }
 
 // part layout: [T, H, splits, M, 2 + dv]: running max, denominator, sums
@@ -284,7 +344,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
     const int* __restrict__ token_seq, const int* __restrict__ positions, int H,
     int G, int d, int dv, int block_size, int per_page, int window, int P,
     float scale, float softcap, float lam, float norm_eps, float out_mult,
-    int splits, int FL) {
+    int splits, int FL, const float* __restrict__ head_bias,
+    const T* __restrict__ gate, int64_t gate_stride) {
   constexpr int NQ = HB * M;
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -318,10 +379,12 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
   const int nk = nb + (pos - lo + 1);
   const int* bt = block_tables + (int64_t)b * bt_stride;
 
-  float mx[NQ], l[NQ], acc[NQ][4];
+  const bool sig = head_bias != nullptr;
+  float mx[NQ], l[NQ], acc[NQ][4], hb[NQ];
 #pragma unroll
   for (int n = 0; n < NQ; ++n) {
-    mx[n] = -INFINITY;
+    hb[n] = sig ? head_bias[g * rep + min(r0 + n / M, rep - 1)] : 0.f;
+    mx[n] = sig ? 0.f : -INFINITY;
     l[n] = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[n][i] = 0.f;
@@ -377,12 +440,18 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
     for (int n = 0; n < NQ; ++n) {
       float sc = s[n] * scale;
       if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
-      if (!valid) sc = -INFINITY;
-      const float m_new = fmaxf(mx[n], wave_reduce_max(sc));  // finite: key u0 is valid
-      const float p = valid ? expf(sc - m_new) : 0.f;
-      corr[n] = expf(mx[n] - m_new);  // exp(-inf) = 0 on the first tile
-      l[n] = l[n] * corr[n] + wave_reduce_sum(p);
-      mx[n] = m_new;
+      float p;
+      if (sig) {
+        p = valid ? ra_sigmoid(sc + hb[n]) : 0.f;
+        corr[n] = 1.0f;
+      } else {
+        if (!valid) sc = -INFINITY;
+        const float m_new = fmaxf(mx[n], wave_reduce_max(sc));  // finite: key u0 is valid
+        p = valid ? expf(sc - m_new) : 0.f;
+        corr[n] = expf(mx[n] - m_new);  // exp(-inf) = 0 on the first tile
+        l[n] = l[n] * corr[n] + wave_reduce_sum(p);
+        mx[n] = m_new;
+      }
       ps[n * 64 + lane] = p;
     }
     rows[lane] = pooled ? -(off + 1) : off;
@@ -483,12 +552,13 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
       float a = 0.f, x = wm[n];
       for (int w = 0; w < RA_WAVES; ++w) a += wl[w * NQ + n];
       for (int w = 1; w < RA_WAVES; ++w) x = fmaxf(x, wm[w * NQ + n]);
-      lg[m] = a;
+      lg[m] = sig ? 1.0f : a;
       mg[m] = x;
     }
     if (splits == 1) {
       ra_epilogue<T, M>(out + (t * H + h) * (int64_t)dv, oacc + hh * M * dvp, dvp,
-                        lg, dv, lam, norm_eps, out_mult);
+                        lg, dv, lam, norm_eps, out_mult,
+                        ra_gate<T>(gate, gate_stride, t, h));
     } else {
 #pragma unroll
       for (int m = 0; m < M; ++m) {
@@ -509,7 +579,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 template <typename T, int M>
 __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
     T* __restrict__ out, const float* __restrict__ part, int dv, int splits,
-    float lam, float norm_eps, float out_mult) {
+    float lam, float norm_eps, float out_mult, int H, int sig,
+    const T* __restrict__ gate, int64_t gate_stride) {
   extern __shared__ float lds[];  // [M][dvp] sums | [M][64] weights
   const int64_t th = blockIdx.x;
   const int lane = threadIdx.x;
@@ -525,6 +596,7 @@ __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
     const float mg = wave_reduce_max(ms);
     const float w = (ms == -INFINITY) ? 0.f : expf(ms - mg);
     lg[m] = wave_reduce_sum(ls * w);
+    if (sig) lg[m] = 1.0f;  // sigmoid weights: the shares' sums add up as they are
     wts[m * 64 + lane] = w;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -553,7 +625,7 @@ __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   ra_epilogue<T, M>(out + th * (int64_t)dv, lds, dvp, lg, dv, lam, norm_eps,
-                    out_mult);
+                    out_mult, ra_gate<T>(gate, gate_stride, th / H, (int)(th % H)));
 }
 
 struct RaArgs {
@@ -569,6 +641,9 @@ struct RaArgs {
   int T_, H, G, d, dv, block_size, per_page, window, P;
   float scale, softcap, lam, norm_eps, out_mult;
   int splits;
+  const float* head_bias;
+  const void* gate;
+  int64_t gate_stride;
   hipStream_t stream;
 };
 
@@ -592,7 +667,8 @@ static void launch_ra_hb(const RaArgs& a) {
                      a.pool, a.block_tables, a.bt_stride, a.token_seq,        \
                      a.positions, a.H, a.G, a.d, a.dv, a.block_size,          \
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,    \
-                     a.norm_eps, a.out_mult, a.splits, FL)
+                     a.norm_eps, a.out_mult, a.splits, FL, a.head_bias,       \
+                     (const T*)a.gate, a.gate_stride)
   if (vec) RA_CALL(true);
   else RA_CALL(false);
 #undef RA_CALL
@@ -600,7 +676,8 @@ static void launch_ra_hb(const RaArgs& a) {
     hipLaunchKernelGGL((row_attention_reduce_kernel<T, M>),
                        dim3(a.T_ * a.H), dim3(64), sizeof(float) * M * (dvp + 64),
                        a.stream, (T*)a.out, a.part, a.dv, a.splits, a.lam,
-                       a.norm_eps, a.out_mult);
+                       a.norm_eps, a.out_mult, a.H, a.head_bias != nullptr,
+                       (const T*)a.gate, a.gate_stride);
 }
 
 template <typename T, int M>
@@ -621,12 +698,14 @@ extern "C" void launch_row_attention(
     const int* block_tables, int bt_stride, const int* token_seq,
     const int* positions, int T_, int H, int G, int M, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
-    float lam, float norm_eps, float out_mult, int splits, int kind,
+    float lam, float norm_eps, float out_mult, int splits,
+    const float* head_bias, const void* gate, int64_t gate_stride, int kind,
     hipStream_t stream) {
   if (T_ == 0) return;
   const RaArgs a{out, part, q, cache, pool, block_tables, bt_stride, token_seq,
                  positions, T_, H, G, d, dv, block_size, per_page, window, P,
-                 scale, softcap, lam, norm_eps, out_mult, splits, stream};
+                 scale, softcap, lam, norm_eps, out_mult, splits, head_bias,
+                 gate, gate_stride, stream};
   if (kind == 0) {
     if (M == 1) launch_ra_m<bf16_t, 1>(a);
     else launch_ra_m<bf16_t, 2>(a);

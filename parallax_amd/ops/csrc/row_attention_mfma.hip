@@ -25,8 +25,12 @@
 // Key and value widths are padded with zeros to D and DV (template sizes).
 //
 // The epilogue (a1 - lam a2 for two maps, exchanged through LDS; optional RMS
-// norm over the value width; division by the softmax sum) works on columns,
-// i.e. per lane pair, too.
+// norm over the value width; division by the softmax sum; optional sigmoid
+// gate per (token, head)) works on columns, i.e. per lane pair, too.
+//
+// SIG instantiations replace the softmax by sigmoid(score + head_bias[h])
+// weights that are not normalised over the keys: no running maximum, no
+// rescaling of the accumulators, masked keys weigh 0.
 #include "seq_common.h"
 
 typedef float f32x16v __attribute__((ext_vector_type(16)));
@@ -87,15 +91,22 @@ DEVINL float rm_tanh(float x) {
   return 1.0f - 2.0f * __frcp_rn(__expf(2.0f * x) + 1.0f);
 }
 
+// sigmoid through the same two hardware approximations
+DEVINL float rm_sigmoid(float x) { return __frcp_rn(1.0f + __expf(-x)); }
+// once per (token, head): the library exponential
+DEVINL float rm_sigmoid_exact(float x) { return 1.0f / (1.0f + expf(-x)); }
+
 // D: padded key width (64 | 128), DVB: 32-wide blocks of the padded value width
-template <typename T, int M, int D, int DVB>
+template <typename T, int M, int D, int DVB, bool SIG>
 __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     T* __restrict__ out, const float* __restrict__ q, const T* __restrict__ cache,
     const float* __restrict__ pool, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ cu, int B,
     const int* __restrict__ positions, int H, int G, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
-    float lam, float norm_eps, float out_mult) {
+    float lam, float norm_eps, float out_mult,
+    const float* __restrict__ head_bias, const T* __restrict__ gate,
+    int64_t gate_stride) {
   constexpr int DV = DVB * 32;
   constexpr int KS = D + RM_PAD, VS = DV + RM_PAD;
   constexpr int HW = 4 / M;  // heads per workgroup
@@ -155,6 +166,7 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
   float mx = -INFINITY, l = 0.f;
   const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  const float hbias = SIG ? head_bias[h] : 0.f;
 
   // staging role: 8 threads per key row, 8 features each at a time
   const int srow = threadIdx.x >> 3, ssub = threadIdx.x & 7;
@@ -285,6 +297,34 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     const bool interior = nq == RM_Q && u0 >= nb && u0 + RM_K <= nk &&
                           jt0 + RM_K - 1 <= p0 && (window == 0 || p_last - jt0 < window);
     float tmax = -INFINITY;
+    float corr = 1.f;
+    if (SIG) {
+      if (interior) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float sc = S[i] * scale;
+          if (softcap > 0.f) sc = softcap * rm_tanh(sc * inv_cap);
+          S[i] = rm_sigmoid(sc + hbias);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int u = u0 + 8 * i + 4 * half + j;
+            bool vis;
+            if (u < nb) {
+              vis = u * P + P - 1 <= pq - window;
+            } else {
+              const int jt = lo + (u - nb);
+              vis = jt <= pq && (window == 0 || pq - jt < window);
+            }
+            float sc = S[4 * i + j] * scale;
+            if (softcap > 0.f) sc = softcap * rm_tanh(sc * inv_cap);
+            S[4 * i + j] = (vis && qvalid && u < nk) ? rm_sigmoid(sc + hbias) : 0.f;
+          }
+      }
+    } else {
     if (interior) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -315,7 +355,7 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float m_new = fmaxf(mx, tmax);
-    float corr = 1.f, psum = 0.f;
+    float psum = 0.f;
     if (m_new == -INFINITY) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) S[i] = 0.f;
@@ -331,11 +371,14 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     psum += __shfl_xor(psum, 32, 64);
     l = l * corr + psum;
     mx = m_new;
+    }  // !SIG
     // ---- O^T += V_tile^T . P^T ------------------------------------------------
 #pragma unroll
     for (int k = 0; k < DVB; ++k) {
+      if (!SIG) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[k][i] *= corr;
+        for (int i = 0; i < 16; ++i) acc[k][i] *= corr;
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -348,7 +391,8 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
 
   // ---- epilogue: lane holds O[query col][feature 32 k + 8 i + 4 half + j] --------
   __syncthreads();  // staging area free
-  const float inv = (qvalid && l > 0.f) ? 1.0f / l : 0.f;
+  const float inv = SIG ? (qvalid ? 1.0f : 0.f)
+                        : ((qvalid && l > 0.f) ? 1.0f / l : 0.f);
   if (M == 2) {
     // the second map's wave parks a2 (times lam) in LDS for its head's first wave
     float* X = lds + hh * (DV * (RM_Q + 1));
@@ -387,6 +431,8 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     r = out_mult / sqrtf(ss / (float)dv + norm_eps);
   }
   if (!stream_on || !qvalid) return;
+  if (gate != nullptr)
+    r *= rm_sigmoid_exact(ldf(gate + (int64_t)(t0 + col) * gate_stride + h));
   T* dst = out + ((int64_t)(t0 + col) * H + h) * dv;
 #pragma unroll
   for (int k = 0; k < DVB; ++k)
@@ -409,11 +455,14 @@ struct RmArgs {
   const int* positions;
   int tiles, H, G, d, dv, block_size, per_page, window, P;
   float scale, softcap, lam, norm_eps, out_mult;
+  const float* head_bias;
+  const void* gate;
+  int64_t gate_stride;
   hipStream_t stream;
 };
 
-template <typename T, int M, int D, int DVB>
-static void launch_rm(const RmArgs& a) {
+template <typename T, int M, int D, int DVB, bool SIG>
+static void launch_rm_k(const RmArgs& a) {
   constexpr int DV = DVB * 32;
   const int rep = a.H / a.G;
   const int hw = 4 / M;
@@ -426,17 +475,25 @@ static void launch_rm(const RmArgs& a) {
     static bool raised = false;
     if (!raised) {
       (void)hipFuncSetAttribute(
-          reinterpret_cast<const void*>(&row_attention_prefill_kernel<T, M, D, DVB>),
+          reinterpret_cast<const void*>(&row_attention_prefill_kernel<T, M, D, DVB, SIG>),
           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
       raised = true;
     }
   }
-  hipLaunchKernelGGL((row_attention_prefill_kernel<T, M, D, DVB>), grid,
+  hipLaunchKernelGGL((row_attention_prefill_kernel<T, M, D, DVB, SIG>), grid,
                      dim3(256), shm, a.stream, (T*)a.out, a.q,
                      (const T*)a.cache, a.pool, a.block_tables, a.bt_stride,
                      a.cu, a.B, a.positions, a.H, a.G, a.d, a.dv, a.block_size,
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,
-                     a.norm_eps, a.out_mult);
+                     a.norm_eps, a.out_mult, a.head_bias, (const T*)a.gate,
+                     a.gate_stride);
+}
+
+// sigmoid weights come with one score map only
+template <typename T, int M, int D, int DVB>
+static void launch_rm(const RmArgs& a) {
+  if (M == 1 && a.head_bias != nullptr) launch_rm_k<T, 1, D, DVB, true>(a);
+  else launch_rm_k<T, M, D, DVB, false>(a);
 }
 
 template <typename T, int M, int D>
@@ -464,11 +521,13 @@ extern "C" void launch_row_attention_prefill(
     const int* block_tables, int bt_stride, const int* cu, int B,
     const int* positions, int tiles, int H, int G, int M, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
-    float lam, float norm_eps, float out_mult, int kind, hipStream_t stream) {
+    float lam, float norm_eps, float out_mult, const float* head_bias,
+    const void* gate, int64_t gate_stride, int kind, hipStream_t stream) {
   if (tiles == 0) return;
   const RmArgs a{out, q, cache, pool, block_tables, bt_stride, cu, B, positions,
                  tiles, H, G, d, dv, block_size, per_page, window, P, scale,
-                 softcap, lam, norm_eps, out_mult, stream};
+                 softcap, lam, norm_eps, out_mult, head_bias, gate, gate_stride,
+                 stream};
   if (kind == 0) {
     if (M == 1) launch_rm_m<bf16_t, 1>(a);
     else launch_rm_m<bf16_t, 2>(a);

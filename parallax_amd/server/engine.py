@@ -408,7 +408,9 @@ class Engine:
             # measured 270 ms p50 TPOT at request-rate 16 from those stalls
             os.environ["PARALLAX_LT_TUNE_MS"] = "0"
         if self.graph_runner is not None:
-            self.graph_runner.capture_all()
+            # as in step(): graphs are captured and replayed in inference mode
+            with torch.inference_mode():
+                self.graph_runner.capture_all()
 
     def set_grammar_vocab(self, vocab: List[str]) -> None:
         """Enable json_schema constrained decoding: vocab[i] is token i's

@@ -5,7 +5,7 @@
 The built .so files land at parallax_amd/ops/_C.*.so (attention, GEMM, MoE,
 sampler kernels) and parallax_amd/ops/_mix.*.so (sequence mixers: fp32-residual
 layer norm, sliding-window latent attention, gated linear attention, sandwich
-RMS norm, row-cache attention). Both are
+RMS norm, row-cache attention, post-norm residual step, minGRU). Both are
 git-ignored; they travel to the GPU box with the gpurun snapshot.
 PARALLAX_EXT=_mix (or _C) builds one of them only.
 """
@@ -53,6 +53,7 @@ mix_sources = [
     os.path.join(CSRC, "sandwich_norm.hip"),
     os.path.join(CSRC, "row_attention.hip"),
     os.path.join(CSRC, "row_attention_mfma.hip"),
+    os.path.join(CSRC, "post_norm.hip"),
 ]
 
 wanted = [x for x in os.environ.get("PARALLAX_EXT", "_C,_mix").split(",") if x]

@@ -155,3 +155,59 @@ def forward(cfg, w, tokens, return_layers=False):
     if return_layers:
         return logits, torch.stack(streams)
     return logits
+
+
+def random_weights(cfg, seed=0):
+    """Random weights for a config, rounded to bfloat16 (what a checkpoint
+    holds) and returned in float64."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = int(cfg["width"]), int(cfg["vocab"])
+    w = {}
+
+    def mat(name, rows, cols, scale=1.0):
+        w[name] = torch.randn(rows, cols, generator=g) * (scale / math.sqrt(cols))
+
+    def vec(name, n, mean=0.0, std=1.0):
+        w[name] = mean + std * torch.randn(n, generator=g)
+
+    mat("embed", V, W, math.sqrt(W))
+    vec("embed.norm", W, 1.0, 0.2)
+    vec("final.norm", W, 1.0, 0.2)
+    for i, sp in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        vec(p + "norm1", W, 1.0, 0.2)
+        lf, rt = sp["mixer"]["left"], sp["mixer"]["right"]
+        H, G = int(lf["heads"]), int(lf.get("kv_heads", lf["heads"]))
+        d, dv = int(lf["dim"]), int(lf["vdim"])
+        mat(p + "mix.left.q", H * d, W, 2.0)
+        mat(p + "mix.left.k", G * d, W, 2.0)
+        mat(p + "mix.left.v", G * dv, W)
+        vec(p + "mix.left.q.norm", d, 1.0, 0.3)
+        vec(p + "mix.left.k.norm", d, 1.0, 0.3)
+        vec(p + "mix.left.pb", H, -1.0, 1.0)
+        mat(p + "mix.left.g", H, W, 2.0)
+        mat(p + "mix.left.o", W, H * dv)
+        R = int(rt["width"])
+        mat(p + "mix.right.z", R, W, 2.0)
+        vec(p + "mix.right.z.b", R, 0.0, 1.0)
+        mat(p + "mix.right.x", R, W, 2.0)
+        vec(p + "mix.right.x.b", R, 0.0, 0.5)
+        mat(p + "mix.right.g", R, W, 2.0)
+        mat(p + "mix.right.o", W, R)
+        mlp = sp.get("mlp")
+        if mlp is None:
+            continue
+        vec(p + "norm2", W, 1.0, 0.2)
+        if mlp.get("kind", "moe" if "router" in mlp else "dense") == "dense":
+            ff = int(mlp["ff"])
+            mat(p + "mlp.gate", ff, W, 2.0)
+            mat(p + "mlp.up", ff, W, 2.0)
+            mat(p + "mlp.down", W, ff)
+        else:
+            ff = int(mlp["expert"]["ff"])
+            mat(p + "mlp.router", int(mlp["router"]["experts"]), W, 2.0)
+            for e in range(int(mlp["router"]["experts"])):
+                mat(f"{p}mlp.e{e}.gate", ff, W, 3.0)
+                mat(f"{p}mlp.e{e}.up", ff, W, 3.0)
+                mat(f"{p}mlp.e{e}.down", W, ff)
+    return {k: v.to(torch.bfloat16).to(F64) for k, v in w.items()}
