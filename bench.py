@@ -263,6 +263,53 @@ def qwen3_like_config(z: dict) -> dict:
     }
 
 
+# `--design-compare --design-pair zabusun`: a Zabusun stack (sigmoid-weighted
+# grouped attention beside a minGRU in every layer, post-norm fp32 stream,
+# clamped gated linear units as routed experts weighted on their input, a
+# dense one in the first layer) beside a Qwen3-MoE-style stack (grouped-query
+# softmax attention with q/k norm, routed gated experts) of EQUAL sizes.
+
+ZABUSUN_SIZES = {
+    "s": dict(width=1024, layers=8, heads=16, kv_heads=4, dim=64, gru=1024,
+              experts=16, top=2, ff=512, dense_ff=2048, vocab=32000),
+    "m": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, gru=2048,
+              experts=32, top=4, ff=1024, dense_ff=4096, vocab=32000),
+}
+
+
+def zabusun_config(z: dict) -> dict:
+    moe = {"kind": "moe", "expert": {"ff": z["ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "top": z["top"]}}
+    dense = {"kind": "dense", "ff": z["dense_ff"], "limit": 7.0}
+    mixer = {
+        "left": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
+                 "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+                 "rot": {"dims": z["dim"] // 2, "base": 1e6,
+                         "scaling": {"factor": 4.0, "original": 4096,
+                                     "fast": 32.0, "slow": 1.0}}},
+        "right": {"width": z["gru"]}, "left_scale": 0.7, "right_scale": 0.7,
+    }
+    layers = [{"type": "parallel", "mixer": mixer, "mlp": dense if i == 0 else moe}
+              for i in range(z["layers"])]
+    return {"architecture": "Zabusun", "layers": layers, "norm": {"eps": 1e-6},
+            "vocab": z["vocab"], "width": z["width"], "logit_scale": 1.0}
+
+
+def qwen3_moe_like_config(z: dict) -> dict:
+    return {
+        "architectures": ["Qwen3MoeForCausalLM"], "model_type": "qwen3_moe",
+        "vocab_size": z["vocab"], "hidden_size": z["width"],
+        "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+        "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"],
+        "intermediate_size": z["dense_ff"], "moe_intermediate_size": z["ff"],
+        "num_experts": z["experts"], "num_experts_per_tok": z["top"],
+        "first_k_dense_replace": 1,
+        "norm_topk_prob": True, "rms_norm_eps": 1e-6, "rope_theta": 1e6,
+        "max_position_embeddings": 16384, "tie_word_embeddings": True,
+        "torch_dtype": "bfloat16",
+    }
+
+
 def design_compare(args) -> None:
     from parallax_amd.models.config import ModelConfig
     from parallax_amd.server.engine import Engine, EngineArgs
@@ -274,6 +321,10 @@ def design_compare(args) -> None:
             z = SOGIDRA_SIZES[size]
             pair = (("sogidra", sogidra_config(z)),
                     ("qwen3-like", qwen3_like_config(z)))
+        elif args.design_pair == "zabusun":
+            z = ZABUSUN_SIZES[size]
+            pair = (("zabusun", zabusun_config(z)),
+                    ("qwen3-moe-like", qwen3_moe_like_config(z)))
         else:
             z = DESIGN_SIZES[size]
             pair = (("vurizen", vurizen_config(z)),
@@ -382,17 +433,19 @@ def main():
                          "throughput of a Vurizen stack beside a DeepSeek-V3-"
                          "style stack of equal sizes (one GPU, random weights)")
     ap.add_argument("--design-pair", default="vurizen",
-                    choices=["vurizen", "sogidra"],
+                    choices=["vurizen", "sogidra", "zabusun"],
                     help="which design --design-compare measures: vurizen "
-                         "beside a DeepSeek-V3-style stack, or sogidra beside "
-                         "a Qwen3-style dense stack")
+                         "beside a DeepSeek-V3-style stack, sogidra beside "
+                         "a Qwen3-style dense stack, or zabusun beside a "
+                         "Qwen3-MoE-style stack")
     ap.add_argument("--design-sizes", default="s,m",
                     help="comma list of " + ",".join(DESIGN_SIZES))
     ap.add_argument("--design-batch", type=int, default=8)
     ap.add_argument("--design-prompt", type=int, default=2048)
     ap.add_argument("--design-only", default="",
                     help="one design of the pair (vurizen | deepseek-like | "
-                         "sogidra | qwen3-like; default: both)")
+                         "sogidra | qwen3-like | zabusun | qwen3-moe-like; "
+                         "default: both)")
     args = ap.parse_args()
     if args.design_compare:
         design_compare(args)

@@ -66,6 +66,10 @@ void launch_clamped_glu(void*, const void*, int64_t, int, int, float, float,
 void launch_mingru_scan(void*, const void*, int64_t, const float*, const float*,
                         float*, const int64_t*, const int*, const int*, int,
                         int, int, hipStream_t);
+void launch_mingru_chunked(void*, float*, float*, const void*, int64_t,
+                           const float*, const float*, float*, const int64_t*,
+                           const int*, const int*, int, int, int, int, int,
+                           hipStream_t);
 }
 
 static hipStream_t cur_stream() {
@@ -646,6 +650,23 @@ void mingru_scan(torch::Tensor out, torch::Tensor zug, torch::Tensor z_bias,
     TORCH_CHECK(cu.numel() == B + 1);
   } else {
     TORCH_CHECK(B == T, "one token per sequence without token bounds");
+  }
+  // long prompt portions: chunks of L tokens side by side (about 64 chunks
+  // for a sequence of average length at most, so that folding the earlier
+  // chunks stays cheap)
+  if (has_cu && T >= 256) {
+    const int per_seq = (T + B - 1) / B;
+    const int L = std::max(64, ((per_seq + 63) / 64 + 7) / 8 * 8);
+    const int tiles = (T + L - 1) / L + B;
+    torch::Tensor carry = torch::empty({(int64_t)tiles, 2, width}, state.options());
+    torch::Tensor init = torch::empty({(int64_t)B, width}, state.options());
+    launch_mingru_chunked(out.data_ptr(), carry.data_ptr<float>(),
+                          init.data_ptr<float>(), zug.data_ptr(), zug.stride(0),
+                          z_bias.data_ptr<float>(), u_bias.data_ptr<float>(),
+                          state.data_ptr<float>(), slots.data_ptr<int64_t>(),
+                          cu.data_ptr<int>(), positions.data_ptr<int>(), B, L,
+                          tiles, width, kind, cur_stream());
+    return;
   }
   launch_mingru_scan(out.data_ptr(), zug.data_ptr(), zug.stride(0),
                      z_bias.data_ptr<float>(), u_bias.data_ptr<float>(),

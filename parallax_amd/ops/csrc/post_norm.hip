@@ -16,9 +16,16 @@
 //                        gate pre-activations of 8 tokens are loaded and
 //                        turned into (z, c, silu(g)) off the dependent chain;
 //                        the chain itself is one fused multiply-add per
-//                        token. Prompt portions and decode steps are the same
-//                        code, so a prompt gives the same state however it
-//                        is cut.
+//                        token.
+//   mingru_chunk_*     : the same recurrence for long prompt portions, cut
+//                        into chunks of L tokens that run side by side: the
+//                        recurrence is affine in the state, so a first
+//                        kernel reduces every chunk to (A, B) with S_out =
+//                        A S_in + B (A = prod(1 - z), B = the chunk run from
+//                        zero), and a second one folds the (A, B) of the
+//                        chunks before its own into S_in and runs its chunk
+//                        for the outputs. Everything fp32; the result
+//                        differs from the serial order by rounding only.
 #include "seq_common.h"
 
 #define PN_MAXV 4  // 256 threads x 4 elements x PN_MAXV = width 4096 in registers
@@ -222,6 +229,43 @@ extern "C" void launch_clamped_glu(void* out, const void* x, int64_t x_stride,
 
 #define MG_CHUNK 8
 
+// one chunk [t0, t1) of one channel from state S; OUT: write S_t silu(g_t).
+// Returns the final state; *decay (when given) gets prod(1 - z_t).
+template <typename T, bool OUT>
+DEVINL float mingru_run(T* __restrict__ out, const T* __restrict__ zug,
+                        int64_t stride, int t0, int t1, int c, int width,
+                        float zb, float ub, float S, float* decay) {
+  float A = 1.0f;
+  for (int t = t0; t < t1; t += MG_CHUNK) {
+    float z[MG_CHUNK], cand[MG_CHUNK], g[MG_CHUNK];
+#pragma unroll
+    for (int i = 0; i < MG_CHUNK; ++i) {
+      const int tt = min(t + i, t1 - 1);
+      const T* r = zug + (int64_t)tt * stride + c;
+      z[i] = ldf(r);
+      cand[i] = ldf(r + width);
+      if (OUT) g[i] = ldf(r + 2 * width);
+    }
+#pragma unroll
+    for (int i = 0; i < MG_CHUNK; ++i) {
+      z[i] = pn_sigmoid(z[i] + zb);
+      const float u = cand[i] + ub;
+      cand[i] = u >= 0.f ? u + 0.5f : pn_sigmoid(u);
+      if (OUT) g[i] = g[i] * pn_sigmoid(g[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < MG_CHUNK; ++i) {
+      if (t + i < t1) {
+        S = fmaf(z[i], cand[i] - S, S);
+        A *= 1.0f - z[i];
+        if (OUT) stf(out + (int64_t)(t + i) * width + c, S * g[i]);
+      }
+    }
+  }
+  if (decay) *decay = A;
+  return S;
+}
+
 // zug [T, 3 width] (row stride free): z | u | g pre-activations. grid
 // (sequences, ceil(width / 256)); cu == nullptr: sequence b is token b.
 template <typename T>
@@ -235,35 +279,102 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
   const int t0 = cu ? cu[b] : b, t1 = cu ? cu[b + 1] : b + 1;
   if (t0 >= t1 || c >= width) return;
   float* sp = state + slots[b] * (int64_t)width + c;
-  float S = positions[t0] == 0 ? 0.f : *sp;
-  const float zb = z_bias[c], ub = u_bias[c];
-  for (int t = t0; t < t1; t += MG_CHUNK) {
-    float z[MG_CHUNK], cand[MG_CHUNK], g[MG_CHUNK];
-#pragma unroll
-    for (int i = 0; i < MG_CHUNK; ++i) {
-      const int tt = min(t + i, t1 - 1);
-      const T* r = zug + (int64_t)tt * stride + c;
-      z[i] = ldf(r);
-      cand[i] = ldf(r + width);
-      g[i] = ldf(r + 2 * width);
-    }
-#pragma unroll
-    for (int i = 0; i < MG_CHUNK; ++i) {
-      z[i] = pn_sigmoid(z[i] + zb);
-      const float u = cand[i] + ub;
-      cand[i] = u >= 0.f ? u + 0.5f : pn_sigmoid(u);
-      g[i] = g[i] * pn_sigmoid(g[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < MG_CHUNK; ++i) {
-      if (t + i < t1) {
-        // (1 - z) S + z c
-        S = fmaf(z[i], cand[i] - S, S);
-        stf(out + (int64_t)(t + i) * width + c, S * g[i]);
-      }
-    }
+  const float S = positions[t0] == 0 ? 0.f : *sp;
+  *sp = mingru_run<T, true>(out, zug, stride, t0, t1, c, width, z_bias[c],
+                            u_bias[c], S, nullptr);
+}
+
+// which (sequence, chunk) a tile is; false past the last one. base: index of
+// the sequence's first tile.
+DEVINL bool mingru_tile(const int* __restrict__ cu, int B, int L, int tile,
+                        int* b_out, int* chunk, int* base) {
+  int b = 0, first = 0;
+  for (; b < B; ++b) {
+    const int nt = (cu[b + 1] - cu[b] + L - 1) / L;
+    if (tile < first + nt) break;
+    first += nt;
   }
-  *sp = S;
+  if (b == B) return false;
+  *b_out = b;
+  *chunk = tile - first;
+  *base = first;
+  return true;
+}
+
+// carry [tiles][2][width]: (A, B) per chunk; init [B][width]: the state every
+// sequence starts this step from (copied here so that no chunk reads the slot
+// after the last chunk has written it)
+template <typename T>
+__global__ __launch_bounds__(256) void mingru_chunk_reduce_kernel(
+    float* __restrict__ carry, float* __restrict__ init,
+    const T* __restrict__ zug, int64_t stride, const float* __restrict__ z_bias,
+    const float* __restrict__ u_bias, const float* __restrict__ state,
+    const int64_t* __restrict__ slots, const int* __restrict__ cu,
+    const int* __restrict__ positions, int B, int L, int width) {
+  int b, chunk, base;
+  if (!mingru_tile(cu, B, L, blockIdx.x, &b, &chunk, &base)) return;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int t0 = cu[b] + chunk * L, t1 = min(t0 + L, cu[b + 1]);
+  if (chunk == 0)
+    init[(int64_t)b * width + c] =
+        positions[t0] == 0 ? 0.f : state[slots[b] * (int64_t)width + c];
+  float A;
+  const float Bv = mingru_run<T, false>(nullptr, zug, stride, t0, t1, c, width,
+                                        z_bias[c], u_bias[c], 0.f, &A);
+  float* dst = carry + (int64_t)blockIdx.x * 2 * width;
+  dst[c] = A;
+  dst[width + c] = Bv;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void mingru_chunk_apply_kernel(
+    T* __restrict__ out, const float* __restrict__ carry,
+    const float* __restrict__ init, const T* __restrict__ zug, int64_t stride,
+    const float* __restrict__ z_bias, const float* __restrict__ u_bias,
+    float* __restrict__ state, const int64_t* __restrict__ slots,
+    const int* __restrict__ cu, int B, int L, int width) {
+  int b, chunk, base;
+  if (!mingru_tile(cu, B, L, blockIdx.x, &b, &chunk, &base)) return;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= width) return;
+  const int t0 = cu[b] + chunk * L, t1 = min(t0 + L, cu[b + 1]);
+  float S = init[(int64_t)b * width + c];
+  const float* cr = carry + (int64_t)base * 2 * width + c;
+#pragma unroll 4
+  for (int k = 0; k < chunk; ++k)
+    S = fmaf(cr[(int64_t)k * 2 * width], S, cr[(int64_t)k * 2 * width + width]);
+  S = mingru_run<T, true>(out, zug, stride, t0, t1, c, width, z_bias[c],
+                          u_bias[c], S, nullptr);
+  if (t1 == cu[b + 1]) state[slots[b] * (int64_t)width + c] = S;
+}
+
+// tiles: an upper bound on the number of chunks (ceil(T / L) + B); carry
+// [tiles, 2, width] and init [B, width] fp32 scratch
+extern "C" void launch_mingru_chunked(void* out, float* carry, float* init,
+                                      const void* zug, int64_t stride,
+                                      const float* z_bias, const float* u_bias,
+                                      float* state, const int64_t* slots,
+                                      const int* cu, const int* positions,
+                                      int B, int L, int tiles, int width,
+                                      int kind, hipStream_t stream) {
+  if (B == 0 || width == 0 || tiles == 0) return;
+  const dim3 grid(tiles, (width + 255) / 256);
+  if (kind == 0) {
+    hipLaunchKernelGGL((mingru_chunk_reduce_kernel<bf16_t>), grid, dim3(256), 0,
+                       stream, carry, init, (const bf16_t*)zug, stride, z_bias,
+                       u_bias, state, slots, cu, positions, B, L, width);
+    hipLaunchKernelGGL((mingru_chunk_apply_kernel<bf16_t>), grid, dim3(256), 0,
+                       stream, (bf16_t*)out, carry, init, (const bf16_t*)zug,
+                       stride, z_bias, u_bias, state, slots, cu, B, L, width);
+  } else {
+    hipLaunchKernelGGL((mingru_chunk_reduce_kernel<float>), grid, dim3(256), 0,
+                       stream, carry, init, (const float*)zug, stride, z_bias,
+                       u_bias, state, slots, cu, positions, B, L, width);
+    hipLaunchKernelGGL((mingru_chunk_apply_kernel<float>), grid, dim3(256), 0,
+                       stream, (float*)out, carry, init, (const float*)zug,
+                       stride, z_bias, u_bias, state, slots, cu, B, L, width);
+  }
 }
 
 extern "C" void launch_mingru_scan(void* out, const void* zug, int64_t stride,

@@ -49,13 +49,12 @@
 // What a segment passes after its norm: a weight per dimension (shared by the
 // segments) and a rotation of its first rot_dims dimensions by the token's
 // position, dimension i paired with i + rot_dims / 2 at angle pos * freq[i]
-// (fp32), cos and sin times rot_mult.
+// (fp32), cos and sin times rot_mult: the token's (cos, sin) pairs are worked
+// out once per workgroup, in LDS, for all heads.
 struct RaSegOps {
-  const float* w;      // [seg] or null
-  const float* freq;   // [rot_dims / 2] or null
-  float rot_mult;
+  const float* w;       // [seg] or null
+  const float* cs;      // LDS [rot_dims / 2][2]: cos, sin (scaled), or null
   int rot_dims;
-  float pos;
 };
 
 // n elements in segments of `seg`; NORM: every segment divided by its RMS
@@ -63,9 +62,9 @@ struct RaSegOps {
 template <typename TI, typename TO, bool NORM>
 DEVINL void ra_segments(const TI* __restrict__ src, TO* __restrict__ dst, int n,
                         int seg, float eps, float mult, const RaSegOps& so) {
-  if (NORM || so.w != nullptr || so.freq != nullptr) {
+  if (NORM || so.w != nullptr || so.cs != nullptr) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int half = so.freq ? so.rot_dims / 2 : 0;
+    const int half = so.cs ? so.rot_dims / 2 : 0;
     for (int s0 = wave * seg; s0 < n; s0 += RA_WAVES * seg) {
       float r = mult;
       if (NORM) {
@@ -84,10 +83,7 @@ DEVINL void ra_segments(const TI* __restrict__ src, TO* __restrict__ dst, int n,
             u *= so.w[i];
             v *= so.w[i + half];
           }
-          float sn, cs;
-          sincosf(so.pos * so.freq[i], &sn, &cs);
-          sn *= so.rot_mult;
-          cs *= so.rot_mult;
+          const float cs = so.cs[2 * i], sn = so.cs[2 * i + 1];
           stf(dst + s0 + i, u * cs - v * sn);
           stf(dst + s0 + i + half, v * cs + u * sn);
         } else if (i >= 2 * half) {
@@ -116,7 +112,18 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
   float temp = 1.0f;
   if (temp_every > 0)
     temp = 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f);
-  RaSegOps so{q_weight, rot_freq, rot_mult, rot_dims, (float)positions[t]};
+  extern __shared__ float rot_cs[];  // [rot_dims / 2][2]
+  if (rot_freq != nullptr) {
+    const float pos = (float)positions[t];
+    for (int i = threadIdx.x; i < rot_dims / 2; i += 64 * RA_WAVES) {
+      float sn, cs;
+      sincosf(pos * rot_freq[i], &sn, &cs);
+      rot_cs[2 * i] = cs * rot_mult;
+      rot_cs[2 * i + 1] = sn * rot_mult;
+    }
+    __syncthreads();
+  }
+  RaSegOps so{q_weight, rot_freq ? rot_cs : nullptr, rot_dims};
   ra_segments<T, float, NORM>(q + t * q_stride, q_out + t * wq, wq, seg, eps,
                               temp, so);
   if (k == nullptr) return;
@@ -145,20 +152,21 @@ extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
       v_stride, positions, slots, (TT*)cache, wq, wk, wv, seg, eps,          \
       temp_coef, temp_every, q_weight, k_weight, rot_freq, rot_mult, rot_dims
   const bool norm = eps >= 0.f;
+  const size_t shm = rot_freq ? sizeof(float) * rot_dims : 0;
   if (kind == 0) {
     if (norm)
       hipLaunchKernelGGL((qkv_store_kernel<bf16_t, true>), dim3(T_), dim3(256),
-                         0, stream, QS_ARGS(bf16_t));
+                         shm, stream, QS_ARGS(bf16_t));
     else
       hipLaunchKernelGGL((qkv_store_kernel<bf16_t, false>), dim3(T_), dim3(256),
-                         0, stream, QS_ARGS(bf16_t));
+                         shm, stream, QS_ARGS(bf16_t));
   } else {
     if (norm)
       hipLaunchKernelGGL((qkv_store_kernel<float, true>), dim3(T_), dim3(256),
-                         0, stream, QS_ARGS(float));
+                         shm, stream, QS_ARGS(float));
     else
       hipLaunchKernelGGL((qkv_store_kernel<float, false>), dim3(T_), dim3(256),
-                         0, stream, QS_ARGS(float));
+                         shm, stream, QS_ARGS(float));
   }
 #undef QS_ARGS
 }
@@ -262,7 +270,7 @@ template <typename TK, int NQ, bool VEC>
 DEVINL void ra_dot(const TK* __restrict__ key, const float* __restrict__ qs,
                    int dp, int d, float* s) {
   if (VEC) {
-#pragma unroll 2
+#pragma unroll 4
     for (int f = 0; f < d; f += 8) {
       float kv[8];
       ra_load8<TK>(key + f, kv);
@@ -463,7 +471,7 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[n][i] *= corr[n];
     const int cnt = min(64, nk - u0);
-#pragma unroll 4
+#pragma unroll 8
     for (int jj = ks; jj < cnt; jj += kp) {
       const int64_t r = rows[jj];
       float vv[4];

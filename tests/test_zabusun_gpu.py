@@ -27,7 +27,9 @@ def close(got, want, dtype) -> bool:
     same_as_whole() is the sharp bf16 check."""
     if dtype == torch.bfloat16:
         e = U.row_errs(got, want)
-        return bool((e < TOL[dtype]).double().mean() >= 0.85 and e.median() < 0.04)
+        few = e.numel() < 8          # a median of a handful of rows says little
+        return bool((e < TOL[dtype]).double().mean() >= 0.85
+                    and (few or e.median() < 0.04))
     return U.rel_err(got, want) < TOL[dtype]
 
 

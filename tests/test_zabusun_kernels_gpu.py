@@ -79,15 +79,17 @@ def test_clamped_glu(dtype, T, I):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("width", [1, 33, 200, 700])
-def test_mingru_scan(dtype, width):
+@pytest.mark.parametrize("lens", [[37, 20, 1], [700, 333, 1]])
+def test_mingru_scan(dtype, width, lens):
     # three sequences in one packed step: a fresh one, a continued one, a
-    # single token; then single-token rows (decode); slots out of order
-    lens, pos0, slots = [37, 20, 1], [0, 11, 5], [4, 0, 2]
+    # single token (short steps run token-serial, long ones in chunks side by
+    # side); then single-token rows (decode); slots out of order
+    pos0, slots = [0, 11, 5], [4, 0, 2]
     T = sum(lens)
     zug = _rand(T, 3 * width + 6, dtype=dtype, seed=7, scale=2.0)[:, 3:3 + 3 * width]
     zb, ub = _rand(width, seed=8), _rand(width, seed=9, scale=0.5)
     state = _rand(6, width, seed=10)
-    cu = torch.tensor([0, 37, 57, 58], dtype=torch.int32)
+    cu = torch.tensor([0, lens[0], lens[0] + lens[1], T], dtype=torch.int32)
     positions = torch.cat([torch.arange(p, p + n) for p, n in zip(pos0, lens)]).int()
     sl = torch.tensor(slots, dtype=torch.int64)
     rt, at = _tol(dtype)
@@ -96,7 +98,7 @@ def test_mingru_scan(dtype, width):
     got = ops.mingru_scan(zug.to(DEV), zb.to(DEV), ub.to(DEV), sg, sl.to(DEV),
                           cu.to(DEV), positions.to(DEV), dtype)
     torch.testing.assert_close(got.float().cpu(), want.float(), rtol=rt, atol=at)
-    torch.testing.assert_close(sg.cpu(), sr, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(sg.cpu(), sr, rtol=2e-5, atol=2e-5)
     assert torch.equal(sg.cpu()[[1, 3, 5]], state[[1, 3, 5]])
     # decode rows
     z1 = zug[:3]
