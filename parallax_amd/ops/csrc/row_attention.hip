@@ -99,6 +99,35 @@ DEVINL void ra_segments(const TI* __restrict__ src, TO* __restrict__ dst, int n,
   }
 }
 
+// n elements of a token's row into LDS as floats; vec: 16-byte loads (the row
+// starts 16-byte aligned and n is a multiple of 8)
+template <typename T>
+DEVINL void ra_stage(const T* __restrict__ src, float* __restrict__ dst, int n,
+                     bool vec) {
+  if (vec) {
+    for (int i = threadIdx.x * 8; i < n; i += 64 * RA_WAVES * 8) {
+      float v[8];
+      if (sizeof(T) == 2) {
+        const bf16x8 raw = load_bf16x8(src + i);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = bf16x8_get(raw, j);
+      } else {
+        const float4 a = *reinterpret_cast<const float4*>(src + i);
+        const float4 b = *reinterpret_cast<const float4*>(src + i + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+        v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+      }
+      *reinterpret_cast<float4*>(dst + i) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(dst + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < n; i += 64 * RA_WAVES) dst[i] = ldf(src + i);
+  }
+}
+
+// LDS: [rot_dims] cos/sin pairs | [wq + wk] the token's queries and keys as
+// floats when `staged` (they fit): one pass of wide loads, then the segment
+// work runs out of LDS instead of re-reading global memory per segment.
 template <typename T, bool NORM>
 __global__ __launch_bounds__(256) void qkv_store_kernel(
     float* __restrict__ q_out, const T* __restrict__ q, int64_t q_stride,
@@ -107,12 +136,19 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
     const int64_t* __restrict__ slots, T* __restrict__ cache, int wq, int wk,
     int wv, int seg, float eps, float temp_coef, int temp_every,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight,
-    const float* __restrict__ rot_freq, float rot_mult, int rot_dims) {
+    const float* __restrict__ rot_freq, float rot_mult, int rot_dims,
+    int staged, int vec) {
   const int64_t t = blockIdx.x;
   float temp = 1.0f;
   if (temp_every > 0)
     temp = 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f);
   extern __shared__ float rot_cs[];  // [rot_dims / 2][2]
+  float* stage = rot_cs + ((rot_freq ? rot_dims : 0) + 3) / 4 * 4;
+  if (staged) {
+    ra_stage<T>(q + t * q_stride, stage, wq, vec);
+    if (k != nullptr) ra_stage<T>(k + t * k_stride, stage + wq, wk, vec);
+    if (rot_freq == nullptr) __syncthreads();
+  }
   if (rot_freq != nullptr) {
     const float pos = (float)positions[t];
     for (int i = threadIdx.x; i < rot_dims / 2; i += 64 * RA_WAVES) {
@@ -124,14 +160,20 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
     __syncthreads();
   }
   RaSegOps so{q_weight, rot_freq ? rot_cs : nullptr, rot_dims};
-  ra_segments<T, float, NORM>(q + t * q_stride, q_out + t * wq, wq, seg, eps,
-                              temp, so);
+  if (staged)
+    ra_segments<float, float, NORM>(stage, q_out + t * wq, wq, seg, eps, temp, so);
+  else
+    ra_segments<T, float, NORM>(q + t * q_stride, q_out + t * wq, wq, seg, eps,
+                                temp, so);
   if (k == nullptr) return;
   const int64_t slot = slots[t];
   if (slot < 0) return;  // pad row of a captured graph
   T* row = cache + slot * (int64_t)(wk + wv);
   so.w = k_weight;
-  ra_segments<T, T, NORM>(k + t * k_stride, row, wk, seg, eps, 1.0f, so);
+  if (staged)
+    ra_segments<float, T, NORM>(stage + wq, row, wk, seg, eps, 1.0f, so);
+  else
+    ra_segments<T, T, NORM>(k + t * k_stride, row, wk, seg, eps, 1.0f, so);
   const T* vals = v ? v + t * v_stride : k + t * k_stride;
   for (int i = threadIdx.x; i < wv; i += 64 * RA_WAVES) row[wk + i] = vals[i];
 }
@@ -150,9 +192,16 @@ extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
 #define QS_ARGS(TT)                                                          \
   q_out, (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v,       \
       v_stride, positions, slots, (TT*)cache, wq, wk, wv, seg, eps,          \
-      temp_coef, temp_every, q_weight, k_weight, rot_freq, rot_mult, rot_dims
+      temp_coef, temp_every, q_weight, k_weight, rot_freq, rot_mult, rot_dims,  \
+      staged, vec
   const bool norm = eps >= 0.f;
-  const size_t shm = rot_freq ? sizeof(float) * rot_dims : 0;
+  // stage the token's queries and keys in LDS when they fit in 48 KB
+  const int rot_floats = ((rot_freq ? rot_dims : 0) + 3) / 4 * 4;
+  const int staged = (rot_floats + wq + wk) <= 12 * 1024;
+  const int vec = wq % 8 == 0 && wk % 8 == 0 && q_stride % 8 == 0 &&
+                  k_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 &&
+                  (k == nullptr || ((uintptr_t)k % 16) == 0);
+  const size_t shm = sizeof(float) * (rot_floats + (staged ? wq + wk : 0));
   if (kind == 0) {
     if (norm)
       hipLaunchKernelGGL((qkv_store_kernel<bf16_t, true>), dim3(T_), dim3(256),

@@ -115,7 +115,10 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
   float* Vs = lds + M * RM_K * KS;    // [32][VS]
 
   // ---- which 32 tokens: tiles never straddle two sequences ---------------------
-  int tile = blockIdx.x, b = 0;
+  // Workgroups start in index order and a sequence's later tiles see more
+  // keys, so the tiles are dealt from the back: the longest run first and
+  // the short ones fill the tail of the launch.
+  int tile = gridDim.x - 1 - blockIdx.x, b = 0;
   for (; b < B; ++b) {
     const int nt = (cu[b + 1] - cu[b] + RM_Q - 1) / RM_Q;
     if (tile < nt) break;
