@@ -72,9 +72,9 @@ class MinGRU(nn.Module):
     the current token, so the whole portion's gate pre-activations come from
     one GEMM and the recurrence itself is elementwise,
 
-        z_t = sigmoid(W_z h_t + b_z),   u_t = W_x h_t + b_x,
-        c_t = u_t + 1/2 (u_t >= 0)  |  sigmoid(u_t) (u_t < 0),
-        S_t = (1 - z_t) S_(t-1) + z_t c_t,      o_t = S_t * silu(W_g h_t),
+        f_t = sigma(W_z h_t + b_z)            (update gate),
+        p_t = W_x h_t + b_x,   c_t = p_t + 1/2 where p_t >= 0, sigma(p_t) below,
+        S_t = S_(t-1) + f_t (c_t - S_(t-1)),   o_t = S_t * silu(W_g h_t),
 
     followed by the output projection. The state [width] lives in the
     engine's LinearStateCache slots in fp32; gates, candidate and state are

@@ -8,9 +8,9 @@ and Sogidra's, with these pieces:
   grouped heads, q/k norm, partial rotation, a per-head score bias and a
   per-head output gate (row_attention.GatedSigmoidAttention), and a minGRU
   (linear_attention.MinGRU);
-* feed-forward: a clamped gated linear unit, y = g sigmoid(1.702 g) (u + 1)
-  with g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit), either
-  dense or as sigmoid-routed experts whose routing weight (the chosen
+* feed-forward: a clamped gated linear unit: with a = W_gate h cut off above
+  at L and b = W_up h cut off at -L and L, W_down (a sigma(1.702 a) (1 + b)),
+  either dense or as sigmoid-routed experts whose routing weight (the chosen
   expert's own score, not renormalised) multiplies the expert's INPUT;
 * the norm sits on a sublayer's OUTPUT only: x += norm(sublayer(x)); the
   sublayers read the residual stream itself.
@@ -81,8 +81,8 @@ class ParallelMixer(nn.Module):
 
 
 class ClampedGluMLP(nn.Module):
-    """W_down (g sigmoid(alpha g) (u + 1)), g = min(W_gate h, limit),
-    u = clamp(W_up h, -limit, limit)."""
+    """W_down (a sigma(alpha a) (1 + b)) with a = W_gate h cut off above at
+    `limit` and b = W_up h cut off at -limit and +limit."""
 
     alpha = 1.702
 

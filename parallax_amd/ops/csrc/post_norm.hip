@@ -9,19 +9,19 @@
 //                        multiple of 4), so every operand is read once. The
 //                        stream is fp32; y1 has the activation type or fp32
 //                        (fp32 expert sums), y2 the activation type.
-//   clamped_glu        : [gate | up] -> g sigmoid(alpha g) (u + 1) with g =
-//                        min(gate, limit), u = clamp(up, -limit, limit).
-//   mingru_scan        : S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, a
+//   clamped_glu        : [gate | up] -> a sigma(alpha a) (1 + b), a = gate cut
+//                        off above at `limit`, b = up cut off at +-limit.
+//   mingru_scan        : S_t = S_(t-1) + f_t (c_t - S_(t-1)) per channel, a
 //                        thread per (sequence, channel), token-serial. The
 //                        gate pre-activations of 8 tokens are loaded and
-//                        turned into (z, c, silu(g)) off the dependent chain;
+//                        turned into (f, c, silu(g)) off the dependent chain;
 //                        the chain itself is one fused multiply-add per
 //                        token.
 //   mingru_chunk_*     : the same recurrence for long prompt portions, cut
 //                        into chunks of L tokens that run side by side: the
 //                        recurrence is affine in the state, so a first
 //                        kernel reduces every chunk to (A, B) with S_out =
-//                        A S_in + B (A = prod(1 - z), B = the chunk run from
+//                        A S_in + B (A = prod(1 - f), B = the chunk run from
 //                        zero), and a second one folds the (A, B) of the
 //                        chunks before its own into S_in and runs its chunk
 //                        for the outputs. Everything fp32; the result

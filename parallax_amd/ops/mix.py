@@ -303,8 +303,8 @@ def branch_rmsnorm_add(x, y1, y2, a, b, weight, eps, out_dtype, keep_stream=True
 def mingru_scan(zug, z_bias, u_bias, state, slots, cu, positions, out_dtype):
     """minGRU over packed sequences: zug [T, 3 * width] (any row stride) holds
     the pre-activations of update gate, candidate and output gate;
-    S_t = (1 - z) S_(t-1) + z c per channel with z = sigmoid(z_pre + z_bias),
-    c = u + 1/2 for u >= 0, sigmoid(u) otherwise, u = u_pre + u_bias. The fp32
+    S_t = S_(t-1) + f (c - S_(t-1)) per channel with f = sigma(z_pre +
+    z_bias), p = u_pre + u_bias, c = p + 1/2 where p >= 0 and sigma(p) below. The fp32
     state [slots, width] is read (or started from zero at position 0) and
     written back. cu [B+1] int32 token bounds (None: one token each). Returns
     S_t * silu(g_pre) as [T, width] of out_dtype."""
@@ -321,8 +321,9 @@ def mingru_scan(zug, z_bias, u_bias, state, slots, cu, positions, out_dtype):
 
 
 def clamped_glu(gate_up, limit, alpha=1.702):
-    """[gate | up] -> min(gate, limit) * sigmoid(alpha * min(gate, limit)) *
-    (clamp(up, -limit, limit) + 1), fp32 inside, result in the input dtype."""
+    """[gate | up] -> a sigma(alpha a) (1 + b), a = gate cut off above at
+    `limit`, b = up cut off at -limit and +limit; fp32 inside, result in the
+    input dtype."""
     if not gate_up.is_cuda:
         return ref.clamped_glu(gate_up, limit, alpha)
     out = torch.empty(gate_up.shape[0], gate_up.shape[1] // 2,

@@ -861,8 +861,9 @@ def branch_rmsnorm_add(x, y1, y2, a, b, weight, eps, out_dtype, keep_stream=True
 def mingru_scan(zug, z_bias, u_bias, state, slots, cu, positions, out_dtype):
     """minGRU over packed sequences. zug [T, 3 * width]: pre-activations of
     the update gate z, the candidate u and the output gate g of every token.
-      z = sigmoid(z_pre + z_bias),  c = u + 1/2 (u >= 0) | sigmoid(u) (u < 0)
-      with u = u_pre + u_bias,      S_t = (1 - z) S_(t-1) + z c   per channel,
+      f = sigma(z_pre + z_bias),    p = u_pre + u_bias,
+      c = p + 1/2 where p >= 0, sigma(p) below,
+      S_t = S_(t-1) + f (c - S_(t-1))   per channel,
     fp32 throughout; the state [slots, width] fp32 is read (or started from
     zero when the portion begins at position 0) and written back. cu [B+1]
     int32 token bounds (None: one token each). Returns S_t * silu(g_pre) as
@@ -891,8 +892,9 @@ def mingru_scan(zug, z_bias, u_bias, state, slots, cu, positions, out_dtype):
 
 
 def clamped_glu(gate_up, limit, alpha=1.702):
-    """gate_up [T, 2 I] = [gate | up]: g = min(gate, limit), u = clamp(up,
-    -limit, limit); g * sigmoid(alpha * g) * (u + 1) -> [T, I] (fp32 inside)."""
+    """gate_up [T, 2 I] = [gate | up] -> [T, I]: a sigma(alpha a) (1 + b) with
+    a = gate cut off above at `limit`, b = up cut off at -limit and +limit
+    (fp32 inside)."""
     I = gate_up.shape[-1] // 2
     f = gate_up.float()
     g = f[..., :I].clamp(max=limit)
