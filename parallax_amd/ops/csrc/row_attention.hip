@@ -393,7 +393,9 @@ DEVINL float ra_gate(const T* __restrict__ gate, int64_t gate_stride, int64_t t,
 }
 
 // part layout: [T, H, splits, M, 2 + dv]: running max, denominator, sums
-template <typename T, int M, int HB, bool VEC>
+// POOL false: no pooled rows exist, so the value loop has no per-key branch
+// and its loads of several keys are in flight together.
+template <typename T, int M, int HB, bool VEC, bool POOL>
 __global__ __launch_bounds__(256) void row_attention_kernel(
     T* __restrict__ out, float* __restrict__ part, const float* __restrict__ q,
     const T* __restrict__ cache, const float* __restrict__ pool,
@@ -432,7 +434,7 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
   const int b = token_seq ? token_seq[t] : (int)t;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int nb = (window > 0 && P > 0 && pos - window + 1 >= P) ? (pos - window + 1) / P : 0;
+  const int nb = (POOL && window > 0 && P > 0 && pos - window + 1 >= P) ? (pos - window + 1) / P : 0;
   const int nk = nb + (pos - lo + 1);
   const int* bt = block_tables + (int64_t)b * bt_stride;
 
@@ -463,7 +465,7 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 #pragma unroll
     for (int n = 0; n < NQ; ++n) s[n] = 0.f;
     if (valid) {
-      pooled = u < nb;
+      pooled = POOL && u < nb;
       if (pooled) {
         off = ((int64_t)bt[u / per_page] * per_page + u % per_page) * E;
 #pragma unroll
@@ -526,7 +528,7 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
       float vv[4];
       if (VEC) {
         if (fl < dv) {
-          if (r < 0) ra_load4<float>(pool + (-r - 1) + vcol + fl, vv);
+          if (POOL && r < 0) ra_load4<float>(pool + (-r - 1) + vcol + fl, vv);
           else ra_load4<T>(cache + r + vcol + fl, vv);
         } else {
           vv[0] = vv[1] = vv[2] = vv[3] = 0.f;
@@ -535,8 +537,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           const int f = fl + 64 * c;
-          vv[c] = f < dv ? (r < 0 ? pool[(-r - 1) + vcol + f]
-                                  : ldf(cache + r + vcol + f))
+          vv[c] = f < dv ? ((POOL && r < 0) ? pool[(-r - 1) + vcol + f]
+                                            : ldf(cache + r + vcol + f))
                          : 0.f;
         }
       }
@@ -718,16 +720,22 @@ static void launch_ra_hb(const RaArgs& a) {
   const bool vec = (a.d % 8 == 0) && (a.dv % 8 == 0);
   int FL = 1;
   while (FL * 4 < a.dv) FL <<= 1;  // dv <= 256 -> FL <= 64
-#define RA_CALL(V)                                                            \
-  hipLaunchKernelGGL((row_attention_kernel<T, M, HB, V>), grid, dim3(256), shm, \
+#define RA_CALL(V, PL)                                                        \
+  hipLaunchKernelGGL((row_attention_kernel<T, M, HB, V, PL>), grid, dim3(256), shm, \
                      a.stream, (T*)a.out, a.part, a.q, (const T*)a.cache,     \
                      a.pool, a.block_tables, a.bt_stride, a.token_seq,        \
                      a.positions, a.H, a.G, a.d, a.dv, a.block_size,          \
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,    \
                      a.norm_eps, a.out_mult, a.splits, FL, a.head_bias,       \
                      (const T*)a.gate, a.gate_stride)
-  if (vec) RA_CALL(true);
-  else RA_CALL(false);
+  const bool pooled = a.pool != nullptr && a.window > 0 && a.P > 0;
+  if (vec) {
+    if (pooled) RA_CALL(true, true);
+    else RA_CALL(true, false);
+  } else {
+    if (pooled) RA_CALL(false, true);
+    else RA_CALL(false, false);
+  }
 #undef RA_CALL
   if (a.splits > 1)
     hipLaunchKernelGGL((row_attention_reduce_kernel<T, M>),

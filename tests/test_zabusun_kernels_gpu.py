@@ -136,8 +136,11 @@ class _Paged:
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("H,G,d,dv,rot", [(6, 2, 12, 20, 8), (8, 2, 96, 80, 32),
                                           (4, 4, 16, 8, 16), (3, 1, 24, 24, 0),
-                                          (2, 1, 136, 264, 100)])
+                                          (2, 1, 136, 264, 100), (50, 2, 256, 8, 64)])
 def test_qk_norm_rotation_store(dtype, H, G, d, dv, rot):
+    """Rows that are staged in LDS by 16-byte loads (widths in multiples of
+    8), by scalar loads (12 / 20), and rows too wide to stage (50 heads of
+    256)."""
     T, bs = 9, 4
     q = _rand(T, H * d + 8, dtype=dtype, seed=11)[:, 8:]
     k = _rand(T, G * d, dtype=dtype, seed=12, scale=3.0)
