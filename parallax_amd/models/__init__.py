@@ -19,3 +19,4 @@ from . import minimax_m3  # noqa: F401
 from . import vurizen  # noqa: F401
 from . import sogidra  # noqa: F401
 from . import zabusun  # noqa: F401
+from . import pudizen  # noqa: F401

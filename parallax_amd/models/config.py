@@ -13,6 +13,11 @@ from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
 
+# layer-list designs whose every layer keeps one plain cache row per token
+# (no pooled rows, no recurrent state slots, no layer reading another's rows)
+_PLAIN_ROW_DESIGNS = ("Pudizen",)
+
+
 @dataclass
 class ModelConfig:
     architecture: str = "LlamaForCausalLM"
@@ -86,12 +91,16 @@ class ModelConfig:
     linear_value_head_dim: int = 0
     linear_conv_kernel_dim: int = 4
 
-    # -- per-layer stacks (vurizen, sogidra, zabusun): every layer carries its own mixer and
+    # -- per-layer stacks (vurizen, sogidra, zabusun, pudizen): every layer carries its own mixer and
     # feed-forward description; the flat fields above hold the first layer's
     # values only so that sizing helpers have something to read ----------------
     layer_specs: Optional[List[Dict[str, Any]]] = None
     residual_mult: float = 1.0
     logit_scale: float = 1.0         # the logits are multiplied by this
+    norm_groups: int = 1             # RMS norms split the width into this many parts
+    embed_scale: float = 1.0         # the token embedding is multiplied by this
+    # hashed (previous token, token) embedding: {"buckets", "mul_prev", "mul_cur"}
+    pair_hash: Optional[Dict[str, int]] = None
 
     raw: Dict[str, Any] = field(default_factory=dict, repr=False)
 
@@ -116,6 +125,19 @@ class ModelConfig:
         width) over all key/value heads for the row-attention mixers. Layers
         that read another layer's entry (`kv_from`) and layers without a
         paged cache are left out."""
+        if self.layer_specs is not None and self.architecture in _PLAIN_ROW_DESIGNS:
+            # one row [keys | values] per token for the grouped-head mixers,
+            # the latent alone (no rotated key part) for the latent ones
+            dims = []
+            for sp in self.layer_specs[start:end]:
+                mx = sp["mixer"]
+                if sp["type"] == "latent_attention":
+                    dims.append((int(mx["kv_rank"]), 0))
+                else:
+                    g = int(mx.get("kv_heads", mx["heads"]))
+                    dims.append((g * int(mx["dim"]),
+                                 g * int(mx.get("vdim", mx["dim"]))))
+            return dims
         if self.layer_specs is not None:
             dims = []
             for sp in self.layer_specs[start:end]:
@@ -144,7 +166,7 @@ class ModelConfig:
         """For every cache-owning layer of latent_cache_dims(start, end): the
         number of tokens whose mean row the layer also keeps (pooled blocks
         seen beyond a sliding window), 0 for layers that keep none."""
-        if self.layer_specs is None:
+        if self.layer_specs is None or self.architecture in _PLAIN_ROW_DESIGNS:
             return [0] * len(self.latent_cache_dims(start, end))
         out = []
         for sp in self.layer_specs[start:end]:
@@ -160,6 +182,8 @@ class ModelConfig:
     def linear_state_shapes(self, start: int, end: int) -> List[tuple]:
         """(conv-state shape, recurrent-state shape) of every linear-attention
         layer in [start, end)."""
+        if self.layer_specs is not None and self.architecture in _PLAIN_ROW_DESIGNS:
+            return []
         if self.layer_specs is not None:
             shapes = []
             for sp in self.layer_specs[start:end]:
@@ -192,7 +216,8 @@ class ModelConfig:
     def has_linear_layers(self) -> bool:
         """Whether any layer keeps recurrent state in a per-request slot."""
         if self.layer_specs is not None:
-            return any(sp["type"] in ("gla", "parallel") for sp in self.layer_specs)
+            return self.architecture not in _PLAIN_ROW_DESIGNS and any(
+                sp["type"] in ("gla", "parallel") for sp in self.layer_specs)
         return bool(self.layer_types) and "linear_attention" in self.layer_types
 
     def layer_type(self, layer_idx: int) -> str:
@@ -223,7 +248,14 @@ class ModelConfig:
         attention), 'attention_2' (sliding window with pooled blocks)
         (sogidra); 'parallel' (sigmoid attention beside a minGRU, both reading
         the layer's input) (zabusun). Feed-forward kinds: 'moe' (default),
-        'dense'."""
+        'dense'. Pudizen reuses three of the names for mixers of its own:
+        'attention' (softmax, q/k norm over the whole projection, rotated
+        values), 'attention_2' (sliding window, sigmoid key weights),
+        'latent_attention' (no positions, gated); its top level also carries
+        'embedding' {"scale", "bigram": {"buckets", "mul_prev", "mul_cur"}}
+        and 'norm' {"eps", "groups"}."""
+        if cfg["architecture"] in _PLAIN_ROW_DESIGNS:
+            return cls._from_plain_row_config(cfg)
         layers = cfg["layers"]
         kinds = {"gla": "linear_attention", "latent_attention": "latent_attention",
                  "attention": "diff_attention",
@@ -294,6 +326,55 @@ class ModelConfig:
             g = r.get("groups") or {}
             mc.n_group = int(g.get("count", 0))
             mc.topk_group = int(g.get("keep", 0))
+        return mc
+
+    @classmethod
+    def _from_plain_row_config(cls, cfg: Dict[str, Any]) -> "ModelConfig":
+        layers = cfg["layers"]
+        kinds = {"attention": "attention", "attention_2": "sliding_attention",
+                 "latent_attention": "latent_attention"}
+        for sp in layers:
+            if sp["type"] not in kinds:
+                raise ValueError(f"unknown layer type {sp['type']!r}")
+            mlp = sp.get("mlp")
+            if mlp is not None and mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"unknown feed-forward kind {mlp.get('kind')!r}")
+        first = layers[0]["mixer"]
+        emb = cfg.get("embedding") or {}
+        pair = emb.get("bigram")
+        norm = cfg.get("norm") or {}
+        mc = cls(
+            architecture=cfg["architecture"],
+            model_type=str(cfg["architecture"]).lower(),
+            vocab_size=int(cfg["vocab"]),
+            hidden_size=int(cfg["width"]),
+            num_layers=len(layers),
+            num_heads=int(first["heads"]),
+            num_kv_heads=int(first.get("kv_heads", first["heads"])),
+            head_dim=int(first["dim"]),
+            rms_norm_eps=float(norm.get("eps", 1e-5)),
+            max_position_embeddings=int(cfg.get("max_positions", 1 << 20)),
+            layer_types=[kinds[sp["type"]] for sp in layers],
+            eos_token_ids=[],
+            bos_token_id=None,
+            torch_dtype=cfg.get("torch_dtype", "bfloat16"),
+            layer_specs=layers,
+            norm_groups=int(norm.get("groups", 1)),
+            embed_scale=float(emb.get("scale", 1.0)),
+            pair_hash={k: int(pair[k]) for k in ("buckets", "mul_prev", "mul_cur")}
+            if pair else None,
+            raw=cfg,
+        )
+        if mc.hidden_size % mc.norm_groups:
+            raise ValueError(f"width {mc.hidden_size} does not split into "
+                             f"{mc.norm_groups} norm groups")
+        windows = [int(sp["mixer"]["mask"]["size"]) for sp in layers
+                   if (sp["mixer"].get("mask") or {}).get("size")]
+        if windows:
+            mc.sliding_window = windows[0]
+        ffs = [int(sp["mlp"]["ff"]) for sp in layers if sp.get("mlp") is not None]
+        if ffs:
+            mc.intermediate_size = ffs[0]
         return mc
 
     @classmethod

@@ -34,6 +34,10 @@ class ForwardMeta:
     # host-side max of seq_lens (avoids a device sync when picking the
     # flash-decoding partition count)
     max_seq_len: int = 0
+    # [T] int64: the token before each token in its own sequence, -1 for a
+    # sequence's first token (filled for models that set `uses_prev_tokens`:
+    # their embedding reads the pair)
+    prev_ids: Optional[torch.Tensor] = None
     # derived per-token tables for packed-sequence kernels (built on first
     # use, shared by every layer of the forward)
     _token_seq: Optional[torch.Tensor] = None

@@ -1,4 +1,6 @@
-"""Sliding-window attention over a compressed latent cache.
+"""Attention over a compressed latent cache: with a sliding window and a
+rotated key part (LatentWindowAttention), or without positions, over the whole
+context, with an output gate per head (GatedLatentAttention).
 
 Per token the cache holds one row [latent c (RMS-normed) | rotated key part]
 shared by all heads; a head's key is [W_uk c | rotated part] and its value
@@ -86,3 +88,68 @@ class LatentWindowAttention(nn.Module):
         )
         attn = torch.einsum("thr,hvr->thv", out_lat, w_uv).to(x.dtype)
         return self.o_proj(attn.reshape(T, H * self.dv))
+
+
+class GatedLatentAttention(nn.Module):
+    """Latent attention without positions. Per token the cache holds the
+    RMS-normed latent c = norm(W_dkv x) alone; head h has the key W_uk,h c and
+    the value W_uv,h c, the score q_h . k_h * scale, a full causal mask and an
+    ordinary softmax; the head's result is multiplied by sigmoid(w_g,h . x),
+    a gate that reads the mixer's input. Runs absorbed: the queries are folded
+    through W_uk into the latent space (fp32), ops.row_attention treats the
+    latent row as the one shared key AND value row of all heads (scores,
+    softmax and sums fp32), and the weighted latent sum is expanded through
+    W_uv afterwards; the gate, a scalar per head, commutes with that
+    expansion and is applied inside the attention kernel. own_proj False: a
+    caller merges the input projections (widths `proj_sizes`: queries, latent,
+    gate pre-activations) with others of the same input and calls mix()."""
+
+    def __init__(self, hidden_size: int, heads: int, dim: int, value_dim: int,
+                 rank: int, scale: float, norm_eps: float, cache_layer_idx: int,
+                 own_proj: bool = True):
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.rank = heads, dim, value_dim, rank
+        self.scale, self.eps = float(scale), float(norm_eps)
+        self.cache_layer_idx = cache_layer_idx
+        self.proj_sizes = [heads * dim, rank, heads]
+        self.in_proj = MergedColumnParallelLinear(hidden_size, self.proj_sizes) \
+            if own_proj else None
+        self.latent_norm = nn.Parameter(torch.empty(rank), requires_grad=False)
+        self.w_uk = nn.Parameter(torch.empty(heads, dim, rank), requires_grad=False)
+        self.w_uv = nn.Parameter(torch.empty(heads, value_dim, rank), requires_grad=False)
+        self.o_proj = RowParallelLinear(heads * value_dim, hidden_size)
+        self._f32 = None
+
+    def _constants(self, device):
+        if self._f32 is None or self._f32[0].device != device:
+            self._f32 = (self.w_uk.float().contiguous(),
+                         self.w_uv.float().contiguous(),
+                         torch.empty(0, dtype=torch.float32, device=device))
+        return self._f32
+
+    def invalidate_constants(self) -> None:
+        self._f32 = None
+
+    def mix(self, parts, meta: ForwardMeta, out_dtype) -> torch.Tensor:
+        """parts: [q, latent pre-norm, gate pre-activations] of the step's
+        tokens (strided views are fine) -> [T, heads * value_dim]."""
+        q, dkv, gate = parts
+        T, H = q.shape[0], self.heads
+        w_uk, w_uv, no_freq = self._constants(q.device)
+        cache = meta.mla_cache.layer(self.cache_layer_idx)
+        ops.latent_kv_store(dkv, self.latent_norm, self.eps, no_freq, 1.0, 0,
+                            meta.positions, meta.slot_mapping, cache, self.rank)
+        q_lat = torch.einsum("thd,hdr->thr", q.view(T, H, self.dim).float(), w_uk)
+        o_lat = ops.row_attention(
+            q_lat.reshape(T, H * self.rank), cache, None, meta.block_tables,
+            meta.token_seq(), meta.positions, H, 1, 1, self.rank, self.rank,
+            0, 0, self.scale, 0.0, 0.0, None, 1.0, torch.float32,
+            max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
+            gate=gate, shared_kv=True,
+        )
+        attn = torch.einsum("thr,hvr->thv", o_lat.view(T, H, self.rank), w_uv)
+        return attn.to(out_dtype).reshape(T, H * self.vdim)
+
+    def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        parts = self.in_proj.split_output(self.in_proj(x))
+        return self.o_proj(self.mix(parts, meta, x.dtype))

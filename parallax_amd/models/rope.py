@@ -126,6 +126,33 @@ def yarn_ramp_frequencies(
     return out.float(), 0.1 * math.log(factor) + 1.0
 
 
+def wavelength_scaled_frequencies(
+    dims: int,
+    base: float,
+    factor: float = 1.0,
+    low: float = 1.0,
+    high: float = 4.0,
+    original: float = 0.0,
+) -> torch.Tensor:
+    """Per-pair rotation frequencies f_i = base^(-2i/dims), i < dims/2, scaled
+    by wavelength (the Llama 3.1 rule), for kernels that turn positions into
+    angles themselves. With l_i = 2 pi / f_i: pairs with l_i < original / high
+    keep f_i; pairs with l_i > original / low get f_i / factor; between the
+    two, s = (original / l_i - low) / (high - low) blends them as (1 - s) f_i
+    / factor + s f_i. original <= 0 or factor == 1 means no scaling. Computed
+    in float64, returned as fp32."""
+    idx = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * idx / dims)
+    if not original or factor == 1.0:
+        return f.float()
+    lam = 2.0 * math.pi / f
+    s = (original / lam - low) / (high - low) if high != low else torch.ones_like(f)
+    mid = (1.0 - s) * f / factor + s * f
+    out = torch.where(lam < original / high, f,
+                      torch.where(lam > original / low, f / factor, mid))
+    return out.float()
+
+
 def build_rope_cache_for(cfg: ModelConfig, rot_dim: Optional[int] = None) -> torch.Tensor:
     rot = rot_dim or cfg.head_dim
     inv_freq, mscale = compute_inv_freq_and_scale(

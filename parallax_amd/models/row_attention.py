@@ -6,7 +6,7 @@ depend on how its prompt was cut or batched. Queries are prepared in fp32 by
 ops.qkv_store, which also scatters the step's keys and values; scores,
 softmax and the per-head post-processing are fp32.
 
-Three mixers are built on it:
+Four mixers are built on it:
 
 DifferentialAttention — every head has TWO query/key maps over the same
 values. With a1, a2 the two softmax results, o = a1 - lambda * a2, then o is
@@ -31,6 +31,16 @@ learned weight (shared by the heads) and then a rotation by position on their
 first rot_dims dimensions (pairs i, i + rot_dims/2, YaRN frequency ramp);
 full causal mask; head h's result is multiplied by sigmoid(w_g,h . x), an
 output gate that reads the mixer's input.
+
+RotaryRowAttention — a configurable mixer: softmax, or sigmoid(score +
+b_h) key weights; full causal mask or a sliding window; rotation of the
+first rot_dims dimensions of every query and key head in either pairing
+(i with i + rot_dims/2, or 2i with 2i + 1) at frequencies the caller hands
+in; optionally an RMS norm over the WHOLE query projection and the whole key
+projection (before the split into heads) with weights as wide as those; and
+optionally rotated values: the value of position j is turned by j over its
+whole width before it is cached, and a head's result at position i is turned
+back by i, so that the result depends on i - j only.
 
 Any of them may read ANOTHER layer's cache rows (`owns_cache=False`) with
 its own queries. All sizes and constants are constructor arguments.
@@ -228,6 +238,96 @@ class GatedSigmoidAttention(_RowAttentionBase):
             max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
             head_bias=bias, gate=gate,
         )
+
+    def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        parts = self.in_proj.split_output(self.in_proj(x))
+        return self.o_proj(self.mix(parts, meta, x.dtype))
+
+
+class RotaryRowAttention(_RowAttentionBase):
+    maps = 1
+
+    def __init__(self, hidden_size: int, heads: int, kv_heads: int, dim: int,
+                 value_dim: int, scale: float, norm_eps: float,
+                 cache_layer_idx: int, owns_cache: bool = True, *,
+                 rot_dims: int = 0, rot_freq: Optional[torch.Tensor] = None,
+                 rot_interleaved: bool = False, qk_norm_whole: bool = False,
+                 value_rot_freq: Optional[torch.Tensor] = None,
+                 window: int = 0, sigmoid_weights: bool = False,
+                 own_proj: bool = True):
+        super().__init__(hidden_size, heads, kv_heads, dim, value_dim, scale,
+                         norm_eps, cache_layer_idx, owns_cache, False, True,
+                         own_proj=own_proj)
+        if rot_dims % 2 or rot_dims > dim:
+            raise ValueError(f"cannot rotate {rot_dims} of {dim} dimensions")
+        if rot_dims and (rot_freq is None or rot_freq.numel() != rot_dims // 2):
+            raise ValueError("one frequency per rotated pair is needed")
+        if value_rot_freq is not None and (
+                value_dim % 2 or value_rot_freq.numel() != value_dim // 2):
+            raise ValueError("rotated values need an even width and one "
+                             "frequency per pair")
+        if window < 0:
+            raise ValueError("window size must not be negative")
+        self.rot_dims = int(rot_dims)
+        self.rot_interleaved = bool(rot_interleaved)
+        self.window = int(window)
+        self._freq = rot_freq.float().contiguous() if self.rot_dims else None
+        self._vfreq = value_rot_freq.float().contiguous() \
+            if value_rot_freq is not None else None
+        self.qk_norm_whole = bool(qk_norm_whole)
+        if self.qk_norm_whole:
+            self.q_norm = nn.Parameter(torch.empty(heads * dim), requires_grad=False)
+            self.k_norm = nn.Parameter(torch.empty(kv_heads * dim), requires_grad=False)
+        self.sigmoid_weights = bool(sigmoid_weights)
+        if self.sigmoid_weights:
+            self.score_bias = nn.Parameter(torch.empty(heads), requires_grad=False)
+        self._f32 = None
+
+    def invalidate_constants(self) -> None:
+        self._f32 = None
+
+    def _constants(self, device):
+        if self._f32 is None or self._f32[4] != device:
+            def f32(p):
+                return p.detach().float().contiguous().to(device)
+            self._f32 = (
+                f32(self.q_norm) if self.qk_norm_whole else None,
+                f32(self.k_norm) if self.qk_norm_whole else None,
+                f32(self.score_bias) if self.sigmoid_weights else None,
+                (self._freq.to(device) if self._freq is not None else None,
+                 self._vfreq.to(device) if self._vfreq is not None else None),
+                device,
+            )
+        return self._f32
+
+    def mix(self, parts, meta: ForwardMeta, out_dtype) -> torch.Tensor:
+        """parts: the projections [q, (k, v)] of the step's tokens (strided
+        views are fine) -> [T, heads * value_dim]."""
+        q = parts[0]
+        k, v = (parts[1], parts[2]) if self.owns_cache else (None, None)
+        wq, wk, bias, (freq, vfreq), _ = self._constants(q.device)
+        cache = meta.mla_cache.layer(self.cache_layer_idx)
+        q32 = ops.qkv_store(
+            q, k, v, meta.positions, meta.slot_mapping, cache, self.dim,
+            self.eps if self.qk_norm_whole else None, 0.0, 0, q_weight=wq,
+            k_weight=wk, rot_freq=freq, rot_mult=1.0, rot_dims=self.rot_dims,
+            norm_whole=self.qk_norm_whole, rot_interleaved=self.rot_interleaved,
+            v_seg=self.vdim, v_rot_freq=vfreq if self.owns_cache else None)
+        o = ops.row_attention(
+            q32, cache, None, meta.block_tables, meta.token_seq(),
+            meta.positions, self.heads, self.kv_heads, 1, self.dim, self.vdim,
+            self.window, 0, self.scale, 0.0, 0.0, None, 1.0,
+            torch.float32 if vfreq is not None else out_dtype,
+            max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
+            head_bias=bias,
+        )
+        if vfreq is not None:
+            # the weighted sum of values turned by their positions, turned
+            # back by the query's position
+            o = ops.rotate_heads(o.view(-1, self.heads, self.vdim),
+                                 meta.positions, vfreq, self.rot_interleaved,
+                                 -1.0, out_dtype)
+        return o
 
     def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
         parts = self.in_proj.split_output(self.in_proj(x))

@@ -653,13 +653,17 @@ from .mix import (  # noqa: E402,F401
     clamped_glu,
     gated_rmsnorm,
     gla_recurrence,
+    group_rmsnorm_add,
     has_mix_extension,
     latent_kv_store,
     latent_window_attention,
     mingru_scan,
+    pair_hash_embedding,
     pool_cache_update,
     qkv_store,
+    relu_squared,
     rope_rows,
+    rotate_heads,
     row_attention,
     sandwich_rmsnorm,
     xielu,

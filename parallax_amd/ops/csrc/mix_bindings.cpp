@@ -41,23 +41,34 @@ void launch_qkv_store(float*, const void*, int64_t, const void*, int64_t,
                       const void*, int64_t, const int*, const int64_t*, void*,
                       int, int, int, int, float, float, int, const float*,
                       const float*, const float*, float, int, int, int,
-                      hipStream_t);
+                      const float*, int, int, int, hipStream_t);
 void launch_pool_cache_update(const void*, float*, const int*, int, const int*,
                               const int*, const int64_t*, int, int, int, int,
                               int, int, hipStream_t);
 int row_attention_heads_per_group(int);
 int row_attention_prefill_supported(int, int);
-void launch_row_attention_prefill(void*, const float*, const void*, const float*,
-                                  const int*, int, const int*, int, const int*,
-                                  int, int, int, int, int, int, int, int, int,
-                                  int, float, float, float, float, float,
-                                  const float*, const void*, int64_t, int,
-                                  hipStream_t);
-void launch_row_attention(void*, float*, const float*, const void*,
+void launch_row_attention_prefill(void*, float*, const float*, const void*,
+                                  const float*, const int*, int, const int*,
+                                  int, const int*, int, int, int, int, int, int,
+                                  int, int, int, int, float, float, float,
+                                  float, float, const float*, const void*,
+                                  int64_t, int, int, hipStream_t);
+void launch_row_attention(void*, float*, float*, const float*, const void*,
                           const float*, const int*, int, const int*, const int*,
                           int, int, int, int, int, int, int, int, int, int,
                           float, float, float, float, float, int, const float*,
-                          const void*, int64_t, int, hipStream_t);
+                          const void*, int64_t, int, int, hipStream_t);
+void launch_group_rmsnorm_add(float*, const void*, int64_t, const void*,
+                              int64_t, const void*, float, void*, int, int,
+                              int, int, hipStream_t);
+void launch_pair_hash_embedding(float*, const int64_t*, const int64_t*,
+                                const void*, const void*, float, int64_t,
+                                int64_t, int64_t, int64_t, int, int, int,
+                                hipStream_t);
+void launch_relu_squared(void*, const void*, int64_t, int, int, int,
+                         hipStream_t);
+void launch_rotate_heads(void*, const float*, const float*, const int*, int,
+                         int, int, float, int, int, hipStream_t);
 void launch_branch_rmsnorm_add(const float*, float*, const void*, int64_t, int,
                                const void*, int64_t, float, float, const void*,
                                float, void*, int, int, int, hipStream_t);
@@ -376,19 +387,31 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                torch::Tensor cache, int64_t seg, double eps, double temp_coef,
                int64_t temp_every, torch::Tensor q_weight,
                torch::Tensor k_weight, torch::Tensor rot_freq, double rot_mult,
-               int64_t rot_dims) {
+               int64_t rot_dims, bool norm_whole, bool rot_interleaved,
+               torch::Tensor v_rot_freq, int64_t v_seg) {
   const int kind = kind_of(q, "q");
   const bool has_qw = q_weight.numel() > 0, has_kw = k_weight.numel() > 0;
   const bool has_rot = rot_freq.numel() > 0 && rot_dims > 0;
+  const bool has_vrot = v_rot_freq.numel() > 0;
   if (has_qw || has_kw || has_rot)
     TORCH_CHECK(seg > 0 && q.size(1) % seg == 0, "query width / segment");
+  // norm_whole: the RMS runs over the whole row and so do the weights
   if (has_qw) {
     CHECK_F32C(q_weight);
-    TORCH_CHECK(q_weight.numel() == seg, "query norm weight width");
+    TORCH_CHECK(q_weight.numel() == (norm_whole ? q.size(1) : seg),
+                "query norm weight width");
   }
   if (has_kw) {
     CHECK_F32C(k_weight);
-    TORCH_CHECK(k_weight.numel() == seg, "key norm weight width");
+    TORCH_CHECK(k.dim() == 2 &&
+                k_weight.numel() == (norm_whole ? k.size(1) : seg),
+                "key norm weight width");
+  }
+  if (has_vrot) {
+    CHECK_F32C(v_rot_freq);
+    TORCH_CHECK(v.dim() == 2 && v_seg > 0 && v_seg % 2 == 0 &&
+                v.size(1) % v_seg == 0 && v_rot_freq.numel() == v_seg / 2,
+                "rotated value segments");
   }
   if (has_rot) {
     CHECK_F32C(rot_freq);
@@ -434,8 +457,10 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                    has_qw ? q_weight.data_ptr<float>() : nullptr,
                    has_kw ? k_weight.data_ptr<float>() : nullptr,
                    has_rot ? rot_freq.data_ptr<float>() : nullptr,
-                   (float)rot_mult, has_rot ? (int)rot_dims : 0, T, kind,
-                   cur_stream());
+                   (float)rot_mult, has_rot ? (int)rot_dims : 0,
+                   norm_whole ? 1 : 0, rot_interleaved ? 1 : 0,
+                   has_vrot ? v_rot_freq.data_ptr<float>() : nullptr,
+                   has_vrot ? (int)v_seg : 0, T, kind, cur_stream());
 }
 
 // cache [blocks, block, E]; pool [blocks, per_page, E] fp32
@@ -477,7 +502,7 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
                    int64_t P, double scale, double softcap, double lam,
                    double norm_eps, double out_mult, int64_t max_keys,
                    torch::Tensor query_bounds, torch::Tensor head_bias,
-                   torch::Tensor gate) {
+                   torch::Tensor gate, bool shared_kv) {
   const int kind = kind_of(cache, "cache");
   CHECK_F32C(q);
   // head_bias [H] fp32: sigmoid(score + head_bias[h]) weights, not normalised;
@@ -501,11 +526,18 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
   TORCH_CHECK(dv <= 256, "value width above 256 is not supported");
   TORCH_CHECK(d <= 1024, "key width above 1024 is not supported");
   TORCH_CHECK(q.size(1) == H * M * d, "query width");
-  const int E = G * M * d + G * dv;
+  // shared_kv: a row holds the keys only and a kv head's values are its keys
+  if (shared_kv) TORCH_CHECK(M == 1 && d == dv, "shared keys and values");
+  const int vbase = shared_kv ? 0 : (int)(G * M * d);
+  const int E = vbase + G * dv;
   TORCH_CHECK(cache.size(2) == E, "cache row width");
-  TORCH_CHECK(out.is_cuda() && out.scalar_type() == cache.scalar_type() &&
+  // the result has the cache's type, or fp32
+  TORCH_CHECK(out.is_cuda() && (out.scalar_type() == cache.scalar_type() ||
+                                out.scalar_type() == torch::kFloat32) &&
               out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
               out.size(1) == H * dv);
+  float* out32 = (kind == 0 && out.scalar_type() == torch::kFloat32)
+                     ? out.data_ptr<float>() : nullptr;
   TORCH_CHECK(window >= 0 && P >= 0);
   int per_page = 1;
   const bool has_pool = window > 0 && P > 0;
@@ -534,14 +566,15 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
     const int B = query_bounds.numel() - 1;
     TORCH_CHECK(B >= 1 && block_tables.size(0) >= B);
     launch_row_attention_prefill(
-        out.data_ptr(), q.data_ptr<float>(), cache.data_ptr(),
+        out.data_ptr(), out32, q.data_ptr<float>(), cache.data_ptr(),
         has_pool ? pool.data_ptr<float>() : nullptr,
         block_tables.data_ptr<int>(), (int)block_tables.stride(0),
         query_bounds.data_ptr<int>(), B, positions.data_ptr<int>(),
         (T + 31) / 32 + B, (int)H, (int)G, (int)M, (int)d, (int)dv,
         (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
         (float)scale, (float)softcap, (float)lam, (float)norm_eps,
-        (float)out_mult, bias_p, gate_p, gate_stride, kind, cur_stream());
+        (float)out_mult, bias_p, gate_p, gate_stride, vbase, kind,
+        cur_stream());
     return;
   }
   // shares of the key list per token: enough workgroups to fill the chip
@@ -565,14 +598,102 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
   if (splits > 1)
     part = torch::empty({(int64_t)T, H, splits, M, dv + 2}, q.options());
   launch_row_attention(
-      out.data_ptr(), splits > 1 ? part.data_ptr<float>() : nullptr,
+      out.data_ptr(), out32, splits > 1 ? part.data_ptr<float>() : nullptr,
       q.data_ptr<float>(), cache.data_ptr(),
       has_pool ? pool.data_ptr<float>() : nullptr, block_tables.data_ptr<int>(),
       (int)block_tables.stride(0), has_seq ? token_seq.data_ptr<int>() : nullptr,
       positions.data_ptr<int>(), T, (int)H, (int)G, (int)M, (int)d, (int)dv,
       (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
       (float)scale, (float)softcap, (float)lam, (float)norm_eps,
-      (float)out_mult, splits, bias_p, gate_p, gate_stride, kind, cur_stream());
+      (float)out_mult, splits, bias_p, gate_p, gate_stride, vbase, kind,
+      cur_stream());
+}
+
+// x [T, W] fp32 (updated in place when y1 is given); y1, y2 [T, W] of the
+// activation type or empty (row strides free); weight [W] and out [T, W] of
+// the activation type, or both empty (no norm)
+void group_rmsnorm_add(torch::Tensor x, torch::Tensor y1, torch::Tensor y2,
+                       torch::Tensor weight, int64_t groups, double eps,
+                       torch::Tensor out) {
+  CHECK_F32C(x);
+  TORCH_CHECK(x.dim() == 2);
+  const int T = x.size(0), W = x.size(1);
+  const bool has_y1 = y1.numel() > 0, has_y2 = y2.numel() > 0;
+  const bool has_w = weight.numel() > 0;
+  TORCH_CHECK(has_y1 || has_w, "nothing to do");
+  TORCH_CHECK(has_y1 || !has_y2, "y2 without y1");
+  const int kind = kind_of(has_w ? weight : y1, "activation");
+  auto check_y = [&](const torch::Tensor& y) {
+    TORCH_CHECK(y.is_cuda() && kind_of(y, "y") == kind && y.dim() == 2 &&
+                y.size(0) == T && y.size(1) == W && y.stride(1) == 1);
+  };
+  if (has_y1) check_y(y1);
+  if (has_y2) check_y(y2);
+  TORCH_CHECK(groups >= 1 && groups <= 1024 && W % groups == 0,
+              "the width does not split into the norm's groups");
+  if (has_w)
+    TORCH_CHECK(weight.is_cuda() && weight.is_contiguous() &&
+                weight.numel() == W && out.is_cuda() && out.is_contiguous() &&
+                kind_of(out, "out") == kind && out.dim() == 2 &&
+                out.size(0) == T && out.size(1) == W);
+  launch_group_rmsnorm_add(x.data_ptr<float>(),
+                           has_y1 ? y1.data_ptr() : nullptr,
+                           has_y1 ? y1.stride(0) : 0,
+                           has_y2 ? y2.data_ptr() : nullptr,
+                           has_y2 ? y2.stride(0) : 0,
+                           has_w ? weight.data_ptr() : nullptr, (float)eps,
+                           has_w ? out.data_ptr() : nullptr, T, W, (int)groups,
+                           kind, cur_stream());
+}
+
+// out [T, W] fp32; ids, prev [T] int64; table [vocab, W], pair [buckets + 1, W]
+void pair_hash_embedding(torch::Tensor out, torch::Tensor ids,
+                         torch::Tensor prev, torch::Tensor table,
+                         torch::Tensor pair, double scale, int64_t buckets,
+                         int64_t mul_prev, int64_t mul_cur) {
+  const int kind = kind_of(table, "table");
+  CHECK_F32C(out);
+  CHECK_I64(ids);
+  CHECK_I64(prev);
+  const int T = ids.numel(), W = table.size(1);
+  TORCH_CHECK(prev.numel() == T && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == W);
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous() && pair.is_cuda() &&
+              pair.scalar_type() == table.scalar_type() && pair.dim() == 2 &&
+              pair.is_contiguous() && pair.size(1) == W &&
+              pair.size(0) == buckets + 1 && buckets >= 1, "pair table");
+  launch_pair_hash_embedding(out.data_ptr<float>(), ids.data_ptr<int64_t>(),
+                             prev.data_ptr<int64_t>(), table.data_ptr(),
+                             pair.data_ptr(), (float)scale, buckets, mul_prev,
+                             mul_cur, table.size(0), W, T, kind, cur_stream());
+}
+
+// x [rows, I] (row stride free) -> out [rows, I]
+void relu_squared(torch::Tensor out, torch::Tensor x) {
+  const int kind = kind_of(x, "x");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1 && out.is_cuda() &&
+              out.scalar_type() == x.scalar_type() && out.is_contiguous() &&
+              out.dim() == 2 && out.size(0) == x.size(0) &&
+              out.size(1) == x.size(1));
+  launch_relu_squared(out.data_ptr(), x.data_ptr(), x.stride(0), (int)x.size(1),
+                      (int)x.size(0), kind, cur_stream());
+}
+
+// x [T, H, D] fp32 -> out [T, H * D] (bf16 or fp32); freq [D / 2]
+void rotate_heads(torch::Tensor out, torch::Tensor x, torch::Tensor freq,
+                  torch::Tensor positions, bool interleaved, double sign) {
+  const int kind = kind_of(out, "out");
+  CHECK_F32C(x);
+  CHECK_F32C(freq);
+  CHECK_I32(positions);
+  TORCH_CHECK(x.dim() == 3);
+  const int T = x.size(0), H = x.size(1), D = x.size(2);
+  TORCH_CHECK(D % 2 == 0 && freq.numel() == D / 2 && positions.numel() == T);
+  TORCH_CHECK(out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == (int64_t)H * D);
+  launch_rotate_heads(out.data_ptr(), x.data_ptr<float>(),
+                      freq.data_ptr<float>(), positions.data_ptr<int>(), H, D,
+                      interleaved ? 1 : 0, (float)sign, T, kind, cur_stream());
 }
 
 // x_in [T, W] fp32 or empty; x_out [T, W] fp32 or empty (may be x_in); y1
@@ -690,4 +811,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("branch_rmsnorm_add", &branch_rmsnorm_add);
   m.def("clamped_glu", &clamped_glu);
   m.def("mingru_scan", &mingru_scan);
+  m.def("group_rmsnorm_add", &group_rmsnorm_add);
+  m.def("pair_hash_embedding", &pair_hash_embedding);
+  m.def("relu_squared", &relu_squared);
+  m.def("rotate_heads", &rotate_heads);
 }

@@ -52,13 +52,29 @@
 // (fp32), cos and sin times rot_mult: the token's (cos, sin) pairs are worked
 // out once per workgroup, in LDS, for all heads.
 struct RaSegOps {
-  const float* w;       // [seg] or null
+  const float* w;       // [seg] (or the whole row's width when w_full) or null
   const float* cs;      // LDS [rot_dims / 2][2]: cos, sin (scaled), or null
   int rot_dims;
+  bool inter;           // pairs (2i, 2i + 1) instead of (i, i + rot_dims / 2)
+  bool w_full;          // the weight has one entry per element of the row
+  float r_whole;        // > 0: the row's 1 / RMS, used for every segment
 };
 
+// 1 / RMS over all n elements of a row; every thread of the workgroup gets it
+template <typename TI>
+DEVINL float ra_row_rrms(const TI* __restrict__ src, int n, float eps,
+                         float* scratch) {
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += 64 * RA_WAVES) {
+    const float t = ldf(src + i);
+    ss += t * t;
+  }
+  ss = block256_sum(ss, scratch);
+  return 1.0f / sqrtf(ss / (float)n + eps);
+}
+
 // n elements in segments of `seg`; NORM: every segment divided by its RMS
-// (wave per segment), then times mult.
+// (wave per segment), or by the row's when so.r_whole is set; then times mult.
 template <typename TI, typename TO, bool NORM>
 DEVINL void ra_segments(const TI* __restrict__ src, TO* __restrict__ dst, int n,
                         int seg, float eps, float mult, const RaSegOps& so) {
@@ -68,27 +84,34 @@ DEVINL void ra_segments(const TI* __restrict__ src, TO* __restrict__ dst, int n,
     for (int s0 = wave * seg; s0 < n; s0 += RA_WAVES * seg) {
       float r = mult;
       if (NORM) {
-        float ss = 0.f;
-        for (int i = lane; i < seg; i += 64) {
-          const float t = ldf(src + s0 + i);
-          ss += t * t;
+        if (so.r_whole > 0.f) {
+          r = mult * so.r_whole;
+        } else {
+          float ss = 0.f;
+          for (int i = lane; i < seg; i += 64) {
+            const float t = ldf(src + s0 + i);
+            ss += t * t;
+          }
+          ss = wave_reduce_sum(ss);
+          r = mult / sqrtf(ss / (float)seg + eps);
         }
-        ss = wave_reduce_sum(ss);
-        r = mult / sqrtf(ss / (float)seg + eps);
       }
+      const float* w = so.w ? (so.w_full ? so.w + s0 : so.w) : nullptr;
       for (int i = lane; i < seg; i += 64) {
         if (i < half) {
-          float u = ldf(src + s0 + i) * r, v = ldf(src + s0 + i + half) * r;
-          if (so.w) {
-            u *= so.w[i];
-            v *= so.w[i + half];
+          const int iu = so.inter ? 2 * i : i;
+          const int iv = so.inter ? 2 * i + 1 : i + half;
+          float u = ldf(src + s0 + iu) * r, v = ldf(src + s0 + iv) * r;
+          if (w) {
+            u *= w[iu];
+            v *= w[iv];
           }
           const float cs = so.cs[2 * i], sn = so.cs[2 * i + 1];
-          stf(dst + s0 + i, u * cs - v * sn);
-          stf(dst + s0 + i + half, v * cs + u * sn);
+          stf(dst + s0 + iu, u * cs - v * sn);
+          stf(dst + s0 + iv, v * cs + u * sn);
         } else if (i >= 2 * half) {
           float t = ldf(src + s0 + i) * r;
-          if (so.w) t *= so.w[i];
+          if (w) t *= w[i];
           stf(dst + s0 + i, t);
         }
       }
@@ -125,9 +148,14 @@ DEVINL void ra_stage(const T* __restrict__ src, float* __restrict__ dst, int n,
   }
 }
 
-// LDS: [rot_dims] cos/sin pairs | [wq + wk] the token's queries and keys as
-// floats when `staged` (they fit): one pass of wide loads, then the segment
-// work runs out of LDS instead of re-reading global memory per segment.
+// LDS: [rot_dims] cos/sin pairs | [v_seg] cos/sin pairs of the value rotation
+// | [wq + wk] the token's queries and keys as floats when `staged` (they
+// fit): one pass of wide loads, then the segment work runs out of LDS
+// instead of re-reading global memory per segment.
+// whole: the RMS of NORM runs over the whole query row and the whole key row
+// (weights as wide as the rows) instead of per segment. inter: rotation pairs
+// (2i, 2i + 1). v_freq: every v_seg-wide segment of the values is rotated
+// over its whole width by pos * v_freq[m] before it is stored.
 template <typename T, bool NORM>
 __global__ __launch_bounds__(256) void qkv_store_kernel(
     float* __restrict__ q_out, const T* __restrict__ q, int64_t q_stride,
@@ -137,45 +165,68 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
     int wv, int seg, float eps, float temp_coef, int temp_every,
     const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     const float* __restrict__ rot_freq, float rot_mult, int rot_dims,
-    int staged, int vec) {
+    int staged, int vec, int whole, int inter,
+    const float* __restrict__ v_freq, int v_seg) {
+  __shared__ float red[8];
   const int64_t t = blockIdx.x;
   float temp = 1.0f;
   if (temp_every > 0)
     temp = 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every) + 1.0f);
   extern __shared__ float rot_cs[];  // [rot_dims / 2][2]
-  float* stage = rot_cs + ((rot_freq ? rot_dims : 0) + 3) / 4 * 4;
+  float* v_cs = rot_cs + ((rot_freq ? rot_dims : 0) + 3) / 4 * 4;
+  float* stage = v_cs + ((v_freq ? v_seg : 0) + 3) / 4 * 4;
   if (staged) {
     ra_stage<T>(q + t * q_stride, stage, wq, vec);
     if (k != nullptr) ra_stage<T>(k + t * k_stride, stage + wq, wk, vec);
-    if (rot_freq == nullptr) __syncthreads();
   }
+  const float pos = (float)positions[t];
   if (rot_freq != nullptr) {
-    const float pos = (float)positions[t];
     for (int i = threadIdx.x; i < rot_dims / 2; i += 64 * RA_WAVES) {
       float sn, cs;
       sincosf(pos * rot_freq[i], &sn, &cs);
       rot_cs[2 * i] = cs * rot_mult;
       rot_cs[2 * i + 1] = sn * rot_mult;
     }
-    __syncthreads();
   }
-  RaSegOps so{q_weight, rot_freq ? rot_cs : nullptr, rot_dims};
-  if (staged)
+  if (v_freq != nullptr) {
+    for (int i = threadIdx.x; i < v_seg / 2; i += 64 * RA_WAVES) {
+      float sn, cs;
+      sincosf(pos * v_freq[i], &sn, &cs);
+      v_cs[2 * i] = cs;
+      v_cs[2 * i + 1] = sn;
+    }
+  }
+  __syncthreads();
+  const bool full = NORM && whole;
+  RaSegOps so{q_weight, rot_freq ? rot_cs : nullptr, rot_dims, inter != 0,
+              full, 0.f};
+  if (staged) {
+    if (full) so.r_whole = ra_row_rrms<float>(stage, wq, eps, red);
     ra_segments<float, float, NORM>(stage, q_out + t * wq, wq, seg, eps, temp, so);
-  else
+  } else {
+    if (full) so.r_whole = ra_row_rrms<T>(q + t * q_stride, wq, eps, red);
     ra_segments<T, float, NORM>(q + t * q_stride, q_out + t * wq, wq, seg, eps,
                                 temp, so);
+  }
   if (k == nullptr) return;
   const int64_t slot = slots[t];
   if (slot < 0) return;  // pad row of a captured graph
   T* row = cache + slot * (int64_t)(wk + wv);
   so.w = k_weight;
-  if (staged)
+  if (staged) {
+    if (full) so.r_whole = ra_row_rrms<float>(stage + wq, wk, eps, red);
     ra_segments<float, T, NORM>(stage + wq, row, wk, seg, eps, 1.0f, so);
-  else
+  } else {
+    if (full) so.r_whole = ra_row_rrms<T>(k + t * k_stride, wk, eps, red);
     ra_segments<T, T, NORM>(k + t * k_stride, row, wk, seg, eps, 1.0f, so);
+  }
   const T* vals = v ? v + t * v_stride : k + t * k_stride;
-  for (int i = threadIdx.x; i < wv; i += 64 * RA_WAVES) row[wk + i] = vals[i];
+  if (v_freq != nullptr) {
+    const RaSegOps sv{nullptr, v_cs, v_seg, inter != 0, false, 0.f};
+    ra_segments<T, T, false>(vals, row + wk, wv, v_seg, eps, 1.0f, sv);
+  } else {
+    for (int i = threadIdx.x; i < wv; i += 64 * RA_WAVES) row[wk + i] = vals[i];
+  }
 }
 
 extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
@@ -186,17 +237,19 @@ extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
                                  float temp_coef, int temp_every,
                                  const float* q_weight, const float* k_weight,
                                  const float* rot_freq, float rot_mult,
-                                 int rot_dims, int T_, int kind,
-                                 hipStream_t stream) {
+                                 int rot_dims, int whole, int inter,
+                                 const float* v_freq, int v_seg, int T_,
+                                 int kind, hipStream_t stream) {
   if (T_ == 0) return;
 #define QS_ARGS(TT)                                                          \
   q_out, (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v,       \
       v_stride, positions, slots, (TT*)cache, wq, wk, wv, seg, eps,          \
       temp_coef, temp_every, q_weight, k_weight, rot_freq, rot_mult, rot_dims,  \
-      staged, vec
+      staged, vec, whole, inter, v_freq, v_seg
   const bool norm = eps >= 0.f;
   // stage the token's queries and keys in LDS when they fit in 48 KB
-  const int rot_floats = ((rot_freq ? rot_dims : 0) + 3) / 4 * 4;
+  const int rot_floats = ((rot_freq ? rot_dims : 0) + 3) / 4 * 4 +
+                         ((v_freq ? v_seg : 0) + 3) / 4 * 4;
   const int staged = (rot_floats + wq + wk) <= 12 * 1024;
   const int vec = wq % 8 == 0 && wk % 8 == 0 && q_stride % 8 == 0 &&
                   k_stride % 8 == 0 && ((uintptr_t)q % 16) == 0 &&
@@ -352,7 +405,8 @@ DEVINL void ra_dot(const TK* __restrict__ key, const float* __restrict__ qs,
 // unnormalised sums of one head (M maps, acc[m * acc_stride + f], softmax
 // denominators l[m]) into the head's output row.
 template <typename T, int M>
-DEVINL void ra_epilogue(T* __restrict__ dst, const float* __restrict__ acc,
+DEVINL void ra_epilogue(T* __restrict__ dst, float* __restrict__ dst32,
+                        const float* __restrict__ acc,
                         int acc_stride, const float* l, int dv, float lam,
                         float norm_eps, float out_mult, float post) {
   const int lane = threadIdx.x & 63;
@@ -379,7 +433,10 @@ DEVINL void ra_epilogue(T* __restrict__ dst, const float* __restrict__ acc,
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int f = lane + 64 * c;
-    if (f < dv) stf(dst + f, o[c] * r);
+    if (f < dv) {
+      if (dst32) dst32[f] = o[c] * r;
+      else stf(dst + f, o[c] * r);
+    }
   }
 }
 
@@ -397,14 +454,15 @@ DEVINL float ra_gate(const T* __restrict__ gate, int64_t gate_stride, int64_t t,
 // and its loads of several keys are in flight together.
 template <typename T, int M, int HB, bool VEC, bool POOL>
 __global__ __launch_bounds__(256) void row_attention_kernel(
-    T* __restrict__ out, float* __restrict__ part, const float* __restrict__ q,
+    T* __restrict__ out, float* __restrict__ out32, float* __restrict__ part,
+    const float* __restrict__ q,
     const T* __restrict__ cache, const float* __restrict__ pool,
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ token_seq, const int* __restrict__ positions, int H,
     int G, int d, int dv, int block_size, int per_page, int window, int P,
     float scale, float softcap, float lam, float norm_eps, float out_mult,
     int splits, int FL, const float* __restrict__ head_bias,
-    const T* __restrict__ gate, int64_t gate_stride) {
+    const T* __restrict__ gate, int64_t gate_stride, int vbase) {
   constexpr int NQ = HB * M;
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -414,9 +472,10 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
   const int g = blockIdx.y / nhb;
   const int r0 = (blockIdx.y % nhb) * HB;  // first head of the group, within g
   const int split = blockIdx.z;
+  // vbase: the column where a row's values start (0: the values are the keys)
   const int wkeys = G * M * d;
-  const int E = wkeys + G * dv;
-  const int kcol = g * M * d, vcol = wkeys + g * dv;
+  const int E = max(wkeys, vbase + G * dv);
+  const int kcol = g * M * d, vcol = vbase + g * dv;
   const int dp = (d + 7) & ~7;
   const int dvp = (dv + 3) & ~3;
   // LDS: q [NQ][dp] | per wave: p [NQ][64], row offsets [64] (int64)
@@ -615,7 +674,9 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
       mg[m] = x;
     }
     if (splits == 1) {
-      ra_epilogue<T, M>(out + (t * H + h) * (int64_t)dv, oacc + hh * M * dvp, dvp,
+      ra_epilogue<T, M>(out + (t * H + h) * (int64_t)dv,
+                        out32 ? out32 + (t * H + h) * (int64_t)dv : nullptr,
+                        oacc + hh * M * dvp, dvp,
                         lg, dv, lam, norm_eps, out_mult,
                         ra_gate<T>(gate, gate_stride, t, h));
     } else {
@@ -637,7 +698,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
 // features over the splits.
 template <typename T, int M>
 __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
-    T* __restrict__ out, const float* __restrict__ part, int dv, int splits,
+    T* __restrict__ out, float* __restrict__ out32,
+    const float* __restrict__ part, int dv, int splits,
     float lam, float norm_eps, float out_mult, int H, int sig,
     const T* __restrict__ gate, int64_t gate_stride) {
   extern __shared__ float lds[];  // [M][dvp] sums | [M][64] weights
@@ -683,12 +745,15 @@ __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  ra_epilogue<T, M>(out + th * (int64_t)dv, lds, dvp, lg, dv, lam, norm_eps,
+  ra_epilogue<T, M>(out + th * (int64_t)dv,
+                    out32 ? out32 + th * (int64_t)dv : nullptr, lds, dvp, lg,
+                    dv, lam, norm_eps,
                     out_mult, ra_gate<T>(gate, gate_stride, th / H, (int)(th % H)));
 }
 
 struct RaArgs {
   void* out;
+  float* out32;
   float* part;
   const float* q;
   const void* cache;
@@ -703,6 +768,7 @@ struct RaArgs {
   const float* head_bias;
   const void* gate;
   int64_t gate_stride;
+  int vbase;
   hipStream_t stream;
 };
 
@@ -722,12 +788,13 @@ static void launch_ra_hb(const RaArgs& a) {
   while (FL * 4 < a.dv) FL <<= 1;  // dv <= 256 -> FL <= 64
 #define RA_CALL(V, PL)                                                        \
   hipLaunchKernelGGL((row_attention_kernel<T, M, HB, V, PL>), grid, dim3(256), shm, \
-                     a.stream, (T*)a.out, a.part, a.q, (const T*)a.cache,     \
+                     a.stream, (T*)a.out, a.out32, a.part, a.q,               \
+                     (const T*)a.cache,                                       \
                      a.pool, a.block_tables, a.bt_stride, a.token_seq,        \
                      a.positions, a.H, a.G, a.d, a.dv, a.block_size,          \
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,    \
                      a.norm_eps, a.out_mult, a.splits, FL, a.head_bias,       \
-                     (const T*)a.gate, a.gate_stride)
+                     (const T*)a.gate, a.gate_stride, a.vbase)
   const bool pooled = a.pool != nullptr && a.window > 0 && a.P > 0;
   if (vec) {
     if (pooled) RA_CALL(true, true);
@@ -740,7 +807,8 @@ static void launch_ra_hb(const RaArgs& a) {
   if (a.splits > 1)
     hipLaunchKernelGGL((row_attention_reduce_kernel<T, M>),
                        dim3(a.T_ * a.H), dim3(64), sizeof(float) * M * (dvp + 64),
-                       a.stream, (T*)a.out, a.part, a.dv, a.splits, a.lam,
+                       a.stream, (T*)a.out, a.out32, a.part, a.dv, a.splits,
+                       a.lam,
                        a.norm_eps, a.out_mult, a.H, a.head_bias != nullptr,
                        (const T*)a.gate, a.gate_stride);
 }
@@ -759,18 +827,18 @@ extern "C" int row_attention_heads_per_group(int rep) {
 }
 
 extern "C" void launch_row_attention(
-    void* out, float* part, const float* q, const void* cache, const float* pool,
+    void* out, float* out32, float* part, const float* q, const void* cache, const float* pool,
     const int* block_tables, int bt_stride, const int* token_seq,
     const int* positions, int T_, int H, int G, int M, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
     float lam, float norm_eps, float out_mult, int splits,
-    const float* head_bias, const void* gate, int64_t gate_stride, int kind,
-    hipStream_t stream) {
+    const float* head_bias, const void* gate, int64_t gate_stride, int vbase,
+    int kind, hipStream_t stream) {
   if (T_ == 0) return;
-  const RaArgs a{out, part, q, cache, pool, block_tables, bt_stride, token_seq,
+  const RaArgs a{out, out32, part, q, cache, pool, block_tables, bt_stride, token_seq,
                  positions, T_, H, G, d, dv, block_size, per_page, window, P,
                  scale, softcap, lam, norm_eps, out_mult, splits, head_bias,
-                 gate, gate_stride, stream};
+                 gate, gate_stride, vbase, stream};
   if (kind == 0) {
     if (M == 1) launch_ra_m<bf16_t, 1>(a);
     else launch_ra_m<bf16_t, 2>(a);

@@ -99,14 +99,14 @@ DEVINL float rm_sigmoid_exact(float x) { return 1.0f / (1.0f + expf(-x)); }
 // D: padded key width (64 | 128), DVB: 32-wide blocks of the padded value width
 template <typename T, int M, int D, int DVB, bool SIG>
 __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
-    T* __restrict__ out, const float* __restrict__ q, const T* __restrict__ cache,
+    T* __restrict__ out, float* __restrict__ out32, const float* __restrict__ q, const T* __restrict__ cache,
     const float* __restrict__ pool, const int* __restrict__ block_tables,
     int bt_stride, const int* __restrict__ cu, int B,
     const int* __restrict__ positions, int H, int G, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
     float lam, float norm_eps, float out_mult,
     const float* __restrict__ head_bias, const T* __restrict__ gate,
-    int64_t gate_stride) {
+    int64_t gate_stride, int vbase) {
   constexpr int DV = DVB * 32;
   constexpr int KS = D + RM_PAD, VS = DV + RM_PAD;
   constexpr int HW = 4 / M;  // heads per workgroup
@@ -139,9 +139,10 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
   const int hh = wave / M, m = wave % M;   // this wave's stream
   const bool stream_on = r0 + hh < rep;
   const int h = g * rep + min(r0 + hh, rep - 1);
+  // vbase: the column where a row's values start (0: the values are the keys)
   const int wkeys = G * M * d;
-  const int E = wkeys + G * dv;
-  const int kcol = g * M * d, vcol = wkeys + g * dv;
+  const int E = max(wkeys, vbase + G * dv);
+  const int kcol = g * M * d, vcol = vbase + g * dv;
 
   // key list of the tile: pooled blocks [0, nb) then tokens [lo, p_last]
   const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
@@ -436,7 +437,18 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
   if (!stream_on || !qvalid) return;
   if (gate != nullptr)
     r *= rm_sigmoid_exact(ldf(gate + (int64_t)(t0 + col) * gate_stride + h));
-  T* dst = out + ((int64_t)(t0 + col) * H + h) * dv;
+  const int64_t o0 = ((int64_t)(t0 + col) * H + h) * dv;
+  if (out32 != nullptr) {
+#pragma unroll
+    for (int k = 0; k < DVB; ++k)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+        if (f < dv) out32[o0 + f] = acc[k][i] * r;
+      }
+    return;
+  }
+  T* dst = out + o0;
 #pragma unroll
   for (int k = 0; k < DVB; ++k)
 #pragma unroll
@@ -448,6 +460,7 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
 
 struct RmArgs {
   void* out;
+  float* out32;
   const float* q;
   const void* cache;
   const float* pool;
@@ -461,6 +474,7 @@ struct RmArgs {
   const float* head_bias;
   const void* gate;
   int64_t gate_stride;
+  int vbase;
   hipStream_t stream;
 };
 
@@ -484,12 +498,12 @@ static void launch_rm_k(const RmArgs& a) {
     }
   }
   hipLaunchKernelGGL((row_attention_prefill_kernel<T, M, D, DVB, SIG>), grid,
-                     dim3(256), shm, a.stream, (T*)a.out, a.q,
+                     dim3(256), shm, a.stream, (T*)a.out, a.out32, a.q,
                      (const T*)a.cache, a.pool, a.block_tables, a.bt_stride,
                      a.cu, a.B, a.positions, a.H, a.G, a.d, a.dv, a.block_size,
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,
                      a.norm_eps, a.out_mult, a.head_bias, (const T*)a.gate,
-                     a.gate_stride);
+                     a.gate_stride, a.vbase);
 }
 
 // sigmoid weights come with one score map only
@@ -520,17 +534,18 @@ extern "C" int row_attention_prefill_supported(int d, int dv) {
 
 // tiles: an upper bound on the number of 32-token tiles (ceil(T / 32) + B)
 extern "C" void launch_row_attention_prefill(
-    void* out, const float* q, const void* cache, const float* pool,
+    void* out, float* out32, const float* q, const void* cache, const float* pool,
     const int* block_tables, int bt_stride, const int* cu, int B,
     const int* positions, int tiles, int H, int G, int M, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
     float lam, float norm_eps, float out_mult, const float* head_bias,
-    const void* gate, int64_t gate_stride, int kind, hipStream_t stream) {
+    const void* gate, int64_t gate_stride, int vbase, int kind,
+    hipStream_t stream) {
   if (tiles == 0) return;
-  const RmArgs a{out, q, cache, pool, block_tables, bt_stride, cu, B, positions,
+  const RmArgs a{out, out32, q, cache, pool, block_tables, bt_stride, cu, B, positions,
                  tiles, H, G, d, dv, block_size, per_page, window, P, scale,
                  softcap, lam, norm_eps, out_mult, head_bias, gate, gate_stride,
-                 stream};
+                 vbase, stream};
   if (kind == 0) {
     if (M == 1) launch_rm_m<bf16_t, 1>(a);
     else launch_rm_m<bf16_t, 2>(a);

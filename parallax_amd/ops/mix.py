@@ -2,7 +2,9 @@
 attention over a compressed latent cache, gated linear attention; sandwich
 RMS norm with depth-weighted averaging, row-cache attention (differential /
 pooled sliding window / sigmoid-weighted with an output gate) and xIELU;
-post-norm residual step, minGRU scan and the clamped gated linear unit.
+post-norm residual step, minGRU scan and the clamped gated linear unit;
+grouped RMS norm over a parallel residual, hashed pair embedding, squared relu
+and the rotation of head rows by position.
 
 GPU tensors go to the hand-written gfx950 kernels of the in-tree extension
 ``parallax_amd.ops._mix`` (bf16 or float32 activations; scores, norms, decays
@@ -175,19 +177,24 @@ def sandwich_rmsnorm(x, y, w_branch, hist, n_hist, dwa, w_next, eps, offset,
 
 def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
               temp_coef, temp_every, q_weight=None, k_weight=None,
-              rot_freq=None, rot_mult=1.0, rot_dims=0):
+              rot_freq=None, rot_mult=1.0, rot_dims=0, norm_whole=False,
+              rot_interleaved=False, v_seg=0, v_rot_freq=None):
     """Queries to fp32 (optionally RMS-normed per seg_dim-wide segment, with
-    a weight [seg_dim] shared by the segments, rotated by position on each
-    segment's first rot_dims dimensions (pairs i, i + rot_dims/2; angles pos *
-    rot_freq[i] in fp32 inside the kernel) and multiplied by a
-    position-dependent temperature); keys (normed, weighted and rotated
-    alike) and values scattered as one row [keys | values] per token into the
-    paged cache. v None: values = the keys before the norm. k None: no
-    store."""
+    a weight [seg_dim] shared by the segments, or, with norm_whole, over the
+    token's whole row with a weight as wide as the row; rotated by position
+    on each segment's first rot_dims dimensions (pairs i, i + rot_dims/2, or
+    2i, 2i + 1 with rot_interleaved; angles pos * rot_freq[i] in fp32 inside
+    the kernel) and multiplied by a position-dependent temperature); keys
+    (normed, weighted and rotated alike) and values scattered as one row
+    [keys | values] per token into the paged cache. v_rot_freq [v_seg / 2]:
+    every v_seg-wide segment of the values is rotated over its whole width
+    (same pairing) before it is stored. v None: values = the keys before the
+    norm. k None: no store."""
     if not q.is_cuda:
         return ref.qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim,
                              norm_eps, temp_coef, temp_every, q_weight,
-                             k_weight, rot_freq, rot_mult, rot_dims)
+                             k_weight, rot_freq, rot_mult, rot_dims,
+                             norm_whole, rot_interleaved, v_seg, v_rot_freq)
     out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     e = _empty(q)
     ef = _empty(q, torch.float32)
@@ -200,6 +207,8 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
         k_weight if k_weight is not None else ef,
         rot_freq if rot_freq is not None else ef, float(rot_mult),
         int(rot_dims) if rot_freq is not None else 0,
+        bool(norm_whole), bool(rot_interleaved),
+        v_rot_freq if v_rot_freq is not None else ef, int(v_seg),
     )
     return out
 
@@ -221,7 +230,8 @@ def pool_cache_update(cache, pool, block_tables, token_seq, positions,
 def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0,
-                  query_bounds=None, head_bias=None, gate=None):
+                  query_bounds=None, head_bias=None, gate=None,
+                  shared_kv=False):
     """Attention of fp32 queries over paged cache rows [keys | values] with
     grouped heads: full causal (window 0) or a sliding window with pooled
     blocks beyond it, optional tanh soft cap, one or two score maps per head
@@ -234,12 +244,15 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
     long key ranges over workgroups. query_bounds [B+1] int32 (prompt portions:
     tokens of sequence b are query_bounds[b] .. query_bounds[b+1], at
     consecutive positions) lets the GPU path tile 32 tokens per workgroup on
-    the fp32 matrix cores. Returns [T, heads * vdim] of out_dtype."""
+    the fp32 matrix cores. shared_kv: a cache row holds the keys only and a
+    kv head's values are its keys (one map, vdim == dim). Returns [T, heads *
+    vdim] of out_dtype (the cache's type, or float32)."""
     if not q.is_cuda:
         return ref.row_attention(q, cache, pool, block_tables, token_seq,
                                  positions, heads, kv_heads, maps, dim, vdim,
                                  window, pool_tokens, scale, softcap, lam,
-                                 norm_eps, out_mult, out_dtype, head_bias, gate)
+                                 norm_eps, out_mult, out_dtype, head_bias, gate,
+                                 shared_kv)
     if head_bias is not None and maps != 1:
         raise ValueError("sigmoid key weights take one score map per head")
     out = torch.empty(q.shape[0], heads * vdim, dtype=out_dtype, device=q.device)
@@ -257,7 +270,7 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         query_bounds if query_bounds is not None and token_seq is not None
         else _empty(positions),
         head_bias if head_bias is not None else ef,
-        gate if gate is not None else ef,
+        gate if gate is not None else ef, bool(shared_kv),
     )
     return out
 
@@ -329,4 +342,62 @@ def clamped_glu(gate_up, limit, alpha=1.702):
     out = torch.empty(gate_up.shape[0], gate_up.shape[1] // 2,
                       dtype=gate_up.dtype, device=gate_up.device)
     _mix_ext().clamped_glu(out, gate_up, float(limit), float(alpha))
+    return out
+
+
+# -- grouped RMS norm over a parallel residual, hashed pair embedding, relu^2 ----
+
+
+def group_rmsnorm_add(x, y1, y2, weight, groups, eps, out_dtype):
+    """One step of a residual stream whose sublayers all read one norm: x
+    [T, W] fp32 <- x + (y1 + y2) in place (y1 None: no update; y2 None: y1
+    alone), then the RMS norm in `groups` equal consecutive parts times weight
+    -> [T, W] of out_dtype (weight None: no norm, returns None)."""
+    if not x.is_cuda:
+        return ref.group_rmsnorm_add(x, y1, y2, weight, groups, eps, out_dtype)
+    e = _empty(x, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) \
+        if weight is not None else e
+    _mix_ext().group_rmsnorm_add(
+        x, y1 if y1 is not None else e, y2 if y2 is not None else e,
+        weight if weight is not None else e, int(groups), float(eps), out,
+    )
+    return out if weight is not None else None
+
+
+def pair_hash_embedding(ids, prev_ids, table, scale, pair_table, buckets,
+                        mul_prev, mul_cur):
+    """fp32 [T, W]: table[id] * scale + pair_table[(prev * mul_prev + id *
+    mul_cur) mod buckets], or pair_table[buckets] (its last row) where a token
+    has no predecessor (prev < 0). ids, prev_ids [T] int64."""
+    if not table.is_cuda:
+        return ref.pair_hash_embedding(ids, prev_ids, table, scale, pair_table,
+                                       buckets, mul_prev, mul_cur)
+    out = torch.empty(ids.shape[0], table.shape[1], dtype=torch.float32,
+                      device=table.device)
+    _mix_ext().pair_hash_embedding(out, ids, prev_ids, table, pair_table,
+                                   float(scale), int(buckets), int(mul_prev),
+                                   int(mul_cur))
+    return out
+
+
+def relu_squared(x):
+    """max(x, 0)^2; x [rows, I] may be a column range of a wider matrix."""
+    if not x.is_cuda:
+        return ref.relu_squared(x)
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    _mix_ext().relu_squared(out, x)
+    return out
+
+
+def rotate_heads(x, positions, freq, interleaved, sign, out_dtype):
+    """x [T, H, D] fp32: every head turned over its whole width by sign * pos
+    * freq[m] (pair m = dimensions m, m + D/2, or 2m, 2m + 1 when interleaved;
+    angles in fp32). Returns [T, H * D] of out_dtype."""
+    if not x.is_cuda:
+        return ref.rotate_heads(x, positions, freq, interleaved, sign, out_dtype)
+    T, H, D = x.shape
+    out = torch.empty(T, H * D, dtype=out_dtype, device=x.device)
+    _mix_ext().rotate_heads(out, x.contiguous(), freq, positions,
+                            bool(interleaved), float(sign))
     return out

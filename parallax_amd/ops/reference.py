@@ -577,17 +577,24 @@ def add_layernorm(resid, y, scale, mult, weight, bias, eps, out_dtype):
     return out.to(out_dtype)
 
 
-def _rotate_rows(x, positions, freq, mult, rot_dims):
-    """x [T, ..., >=rot_dims] fp32; pair (i, i + rot_dims/2)."""
+def _rotate_rows(x, positions, freq, mult, rot_dims, interleaved=False,
+                 sign=1.0):
+    """x [T, ..., >=rot_dims] fp32; pair (i, i + rot_dims/2), or (2i, 2i+1)
+    when interleaved; sign -1 turns the other way."""
     half = rot_dims // 2
     ang = positions.float().unsqueeze(-1) * freq.float()          # [T, half]
     shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
     c = (torch.cos(ang) * mult).view(shape)
-    s = (torch.sin(ang) * mult).view(shape)
-    u, v = x[..., :half], x[..., half:rot_dims]
+    s = (torch.sin(ang) * (mult * sign)).view(shape)
     out = x.clone()
-    out[..., :half] = u * c - v * s
-    out[..., half:rot_dims] = v * c + u * s
+    if interleaved:
+        u, v = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+        out[..., 0:rot_dims:2] = u * c - v * s
+        out[..., 1:rot_dims:2] = v * c + u * s
+    else:
+        u, v = x[..., :half], x[..., half:rot_dims]
+        out[..., :half] = u * c - v * s
+        out[..., half:rot_dims] = v * c + u * s
     return out
 
 
@@ -596,7 +603,9 @@ def latent_kv_store(dkv, norm_w, eps, freq, mult, rot_dims, positions,
     x = dkv.float()
     lat = x[:, :rank]
     lat = lat / torch.sqrt((lat * lat).mean(-1, keepdim=True) + eps) * norm_w.float()
-    kr = _rotate_rows(x[:, rank:], positions, freq, mult, rot_dims)
+    kr = x[:, rank:]
+    if rot_dims > 0:
+        kr = _rotate_rows(kr, positions, freq, mult, rot_dims)
     entry = torch.cat([lat, kr], dim=-1).to(cache.dtype)
     keep = slot_mapping >= 0
     flat = cache.view(-1, cache.shape[-1])
@@ -698,32 +707,45 @@ def _segment_rms(x, seg, eps):
     return (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(T, -1)
 
 
-def _segment_rotate(x, seg, positions, freq, mult, rot_dims):
+def _segment_rotate(x, seg, positions, freq, mult, rot_dims, interleaved=False):
     T = x.shape[0]
     return _rotate_rows(x.view(T, -1, seg), positions, freq, mult,
-                        rot_dims).reshape(T, -1)
+                        rot_dims, interleaved).reshape(T, -1)
 
 
 def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
               temp_coef, temp_every, q_weight=None, k_weight=None,
-              rot_freq=None, rot_mult=1.0, rot_dims=0):
+              rot_freq=None, rot_mult=1.0, rot_dims=0, norm_whole=False,
+              rot_interleaved=False, v_seg=0, v_rot_freq=None):
     """Queries to fp32 (each seg_dim-wide segment divided by its RMS when
-    norm_eps is given, times q_weight [seg_dim] when given; then its first
-    rot_dims dimensions rotated by position, dimension i paired with i +
-    rot_dims / 2 at angle pos * rot_freq[i], cos and sin times rot_mult, when
-    rot_freq is given; multiplied by 1 + temp_coef * ln(floor((pos + 1) /
-    temp_every) + 1) when temp_every > 0), keys (segments normed, weighted by
+    norm_eps is given, times q_weight [seg_dim] when given; with norm_whole
+    the RMS runs over the token's WHOLE query row and q_weight has the row's
+    width; then each segment's first rot_dims dimensions rotated by position,
+    dimension i paired with i + rot_dims / 2 (or 2i with 2i + 1 when
+    rot_interleaved) at angle pos * rot_freq[i], cos and sin times rot_mult,
+    when rot_freq is given; multiplied by 1 + temp_coef * ln(floor((pos + 1)
+    / temp_every) + 1) when temp_every > 0), keys (normed, weighted by
     k_weight and rotated alike) and values into one cache row [keys | values]
-    per token. v None: the values are the keys as they came in, before the
-    norm. k None: nothing is stored (the layer reads another layer's rows).
-    Slot -1 skips the token."""
-    qf = q.float()
-    if norm_eps is not None:
-        qf = _segment_rms(qf, seg_dim, norm_eps)
-    if q_weight is not None:
-        qf = (qf.view(qf.shape[0], -1, seg_dim) * q_weight.float()).reshape(qf.shape)
-    if rot_freq is not None:
-        qf = _segment_rotate(qf, seg_dim, positions, rot_freq, rot_mult, rot_dims)
+    per token. v_rot_freq [v_seg / 2] given: every v_seg-wide segment of the
+    values is rotated by position over its whole width (same pairing, angles
+    pos * v_rot_freq[m]) before it is stored. v None: the values are the keys
+    as they came in, before the norm. k None: nothing is stored (the layer
+    reads another layer's rows). Slot -1 skips the token."""
+
+    def prepare(x, weight):
+        if norm_eps is not None:
+            x = _segment_rms(x, x.shape[1] if norm_whole else seg_dim, norm_eps)
+        if weight is not None:
+            if norm_whole:
+                x = x * weight.float()
+            else:
+                x = (x.view(x.shape[0], -1, seg_dim) * weight.float()).reshape(x.shape)
+        if rot_freq is not None:
+            x = _segment_rotate(x, seg_dim, positions, rot_freq, rot_mult,
+                                rot_dims, rot_interleaved)
+        return x
+
+    qf = prepare(q.float(), q_weight)
     if temp_every > 0:
         p = positions.float()
         temp = 1.0 + temp_coef * torch.log(torch.floor((p + 1.0) / temp_every) + 1.0)
@@ -731,17 +753,24 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
     if k is not None:
         kf = k.float()
         vals = kf if v is None else v.float()
-        if norm_eps is not None:
-            kf = _segment_rms(kf, seg_dim, norm_eps)
-        if k_weight is not None:
-            kf = (kf.view(kf.shape[0], -1, seg_dim) * k_weight.float()).reshape(kf.shape)
-        if rot_freq is not None:
-            kf = _segment_rotate(kf, seg_dim, positions, rot_freq, rot_mult, rot_dims)
+        kf = prepare(kf, k_weight)
+        if v_rot_freq is not None:
+            vals = _segment_rotate(vals, v_seg, positions, v_rot_freq, 1.0,
+                                   v_seg, rot_interleaved)
         entry = torch.cat([kf, vals], dim=-1).to(cache.dtype)
         keep = slot_mapping >= 0
         flat = cache.view(-1, cache.shape[-1])
         flat[slot_mapping[keep]] = entry[keep]
     return qf.contiguous()
+
+
+def rotate_heads(x, positions, freq, interleaved, sign, out_dtype):
+    """x [T, H, D] fp32: every head turned by its token's position over the
+    whole width D (pair m: dimensions m and m + D/2, or 2m and 2m + 1 when
+    interleaved) by sign * pos * freq[m]. Returns [T, H * D] of out_dtype."""
+    T, H, D = x.shape
+    return _rotate_rows(x.float(), positions, freq, 1.0, D, interleaved,
+                        sign).reshape(T, H * D).to(out_dtype)
 
 
 def pool_cache_update(cache, pool, block_tables, token_seq, positions,
@@ -772,9 +801,10 @@ def pool_cache_update(cache, pool, block_tables, token_seq, positions,
 def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, head_bias=None,
-                  gate=None):
+                  gate=None, shared_kv=False):
     """Attention over cache rows [keys (kv_heads x maps x dim) |
-    values (kv_heads x vdim)]. q [T, heads * maps * dim] fp32. window 0: every
+    values (kv_heads x vdim)]; shared_kv: a row holds the keys only and a kv
+    head's values ARE its keys (vdim == dim, one map). q [T, heads * maps * dim] fp32. window 0: every
     key up to the token's position; window > 0: keys j with 0 <= pos - j <
     window plus, when pool_tokens > 0, the pooled row of every block of
     pool_tokens positions that ends at or before pos - window, in the same
@@ -806,7 +836,7 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
             per_page = pool.shape[1]
             rows = torch.cat([pool[bt[b // per_page], b % per_page], rows], 0)
         k = rows[:, :wk].view(-1, G, M, dim)
-        v = rows[:, wk:].view(-1, G, vdim)
+        v = rows[:, (0 if shared_kv else wk):].view(-1, G, vdim)
         s = torch.einsum("grmd,ngmd->grmn", qv[t], k) * scale
         if softcap > 0:
             s = softcap * torch.tanh(s / softcap)
@@ -900,3 +930,43 @@ def clamped_glu(gate_up, limit, alpha=1.702):
     g = f[..., :I].clamp(max=limit)
     u = f[..., I:].clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate_up.dtype)
+
+
+# -- grouped RMS norm over a parallel residual, hashed pair embedding, relu^2 ----
+
+
+def group_rmsnorm_add(x, y1, y2, weight, groups, eps, out_dtype):
+    """One step of a residual stream whose sublayers all read ONE norm:
+      x <- x + (y1 + y2)     (fp32, in place; y1 None: no update; y2 None: y1 only)
+      h = x split into `groups` equal consecutive parts, each divided by its
+          own sqrt(mean(part^2) + eps), the whole times weight
+    Returns h in out_dtype (None when weight is None)."""
+    if y1 is not None:
+        y = y1.float()
+        if y2 is not None:
+            y = y + y2.float()
+        x.add_(y)
+    if weight is None:
+        return None
+    T, W = x.shape
+    v = x.view(T, groups, W // groups)
+    h = (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(T, W)
+    return (h * weight.float()).to(out_dtype)
+
+
+def pair_hash_embedding(ids, prev_ids, table, scale, pair_table, buckets,
+                        mul_prev, mul_cur):
+    """fp32 [T, W]: table[id] * scale + pair_table[r], r = (prev * mul_prev +
+    id * mul_cur) mod buckets, or r = buckets (the table's last row) where a
+    token has no predecessor (prev < 0)."""
+    ids = ids.long()
+    prev = prev_ids.long()
+    r = (prev.clamp(min=0) * int(mul_prev) + ids * int(mul_cur)) % int(buckets)
+    r = torch.where(prev < 0, torch.full_like(r, int(buckets)), r)
+    return table[ids].float() * float(scale) + pair_table[r].float()
+
+
+def relu_squared(x):
+    """max(x, 0)^2 (fp32 inside, result in the input dtype)."""
+    z = x.float().clamp(min=0.0)
+    return (z * z).to(x.dtype)

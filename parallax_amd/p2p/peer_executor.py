@@ -265,7 +265,7 @@ class PeerExecutor:
             chunks = batch.prefill_chunks
             meta, input_ids, _ = self._head_prefill_meta(chunks)
             with torch.inference_mode():
-                hidden = self.model.embed(input_ids).to(self.hidden_dtype)
+                hidden = self._embed(input_ids, meta)
                 hidden = self.model(hidden, meta)
             packets = []
             t = 0
@@ -287,7 +287,7 @@ class PeerExecutor:
             reqs = batch.decode_reqs
             meta, input_ids = self._head_decode_meta(reqs)
             with torch.inference_mode():
-                hidden = self.model.embed(input_ids).to(self.hidden_dtype)
+                hidden = self._embed(input_ids, meta)
                 hidden = self.model(hidden, meta)
             packets = []
             for i, r in enumerate(reqs):
@@ -297,6 +297,11 @@ class PeerExecutor:
                 )
                 packets.append(pkt)
             self._send_forward(packets)
+
+    def _embed(self, input_ids, meta):
+        if meta.prev_ids is not None:
+            return self.model.embed(input_ids, meta.prev_ids).to(self.hidden_dtype)
+        return self.model.embed(input_ids).to(self.hidden_dtype)
 
     def _head_prefill_meta(self, chunks):
         positions, input_ids, slots, btabs, seq_lens, qlens = [], [], [], [], [], []
@@ -311,6 +316,13 @@ class PeerExecutor:
             qlens.append(c.num_tokens)
         meta = self._meta(True, positions, slots, btabs, seq_lens, qlens,
                           rids=[c.req.rid for c in chunks])
+        if getattr(self.model, "uses_prev_tokens", False):
+            prev = []
+            for c in chunks:
+                ids = c.req.prompt_token_ids
+                prev.append(ids[c.start - 1] if c.start > 0 else -1)
+                prev.extend(ids[c.start : c.start + c.num_tokens - 1])
+            meta.prev_ids = torch.tensor(prev, dtype=torch.long, device=self.device)
         return meta, torch.tensor(input_ids, dtype=torch.long, device=self.device), None
 
     def _head_decode_meta(self, reqs):
@@ -326,6 +338,9 @@ class PeerExecutor:
             seq_lens.append(r.total_len)
         meta = self._meta(False, positions, slots, btabs, seq_lens, None,
                           rids=[r.rid for r in reqs])
+        if getattr(self.model, "uses_prev_tokens", False):
+            meta.prev_ids = torch.tensor([r.decode_prev() for r in reqs],
+                                         dtype=torch.long, device=self.device)
         return meta, torch.tensor(input_ids, dtype=torch.long, device=self.device)
 
     # -- non-head -------------------------------------------------------------------------

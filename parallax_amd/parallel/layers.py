@@ -193,3 +193,24 @@ class VocabEmbedding(nn.Module):
 
     def forward(self, input_ids: torch.Tensor) -> torch.Tensor:
         return F.embedding(input_ids, self.weight)
+
+
+class PairHashEmbedding(nn.Module):
+    """Token embedding times `scale`, plus a row of a second table chosen by a
+    hash of the (previous token, token) pair: row (prev * mul_prev + token *
+    mul_cur) mod buckets; a sequence's first token, which has no predecessor
+    (prev < 0), takes the extra last row `buckets`. The sum is fp32."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, buckets: int,
+                 mul_prev: int, mul_cur: int, scale: float = 1.0):
+        super().__init__()
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.scale = float(scale)
+        self.weight = nn.Parameter(torch.empty(vocab_size, hidden_size), requires_grad=False)
+        self.pair = nn.Parameter(torch.empty(self.buckets + 1, hidden_size),
+                                 requires_grad=False)
+
+    def forward(self, input_ids: torch.Tensor, prev_ids: torch.Tensor) -> torch.Tensor:
+        return ops.pair_hash_embedding(input_ids, prev_ids, self.weight,
+                                       self.scale, self.pair, self.buckets,
+                                       self.mul_prev, self.mul_cur)

@@ -133,6 +133,9 @@ class Engine:
         # dtype of the hidden states that enter and leave a shard (designs
         # that keep their residual stream in fp32 say so on the model class)
         self.hidden_dtype = getattr(self.model, "hidden_dtype", None) or args.dtype
+        # models whose embedding reads the (previous token, token) pair get
+        # every token's predecessor in ForwardMeta.prev_ids
+        self.uses_prev_tokens = bool(getattr(self.model, "uses_prev_tokens", False))
         if args.moe_weight_dtype == "fp8":
             from ..models.moe import FusedMoE
 
@@ -593,11 +596,19 @@ class Engine:
                     input_ids, positions, slots, btabs, seq_lens,
                     rids=[r.rid for r in reqs], linear_slots=lin_slots,
                     input_ids_dev=input_dev,
+                    prev_ids=[r.decode_prev() for r in reqs]
+                    if self.uses_prev_tokens else None,
                 )[: len(reqs)]
+            ids_used = None
         else:
             meta, ids = self._build_decode_meta(reqs)
             if input_dev is not None:
                 ids = input_dev.view(-1)[: len(reqs)].to(ids.device, ids.dtype)
+                if self.uses_prev_tokens:
+                    # the host holds a placeholder for the newest token: the
+                    # pair's first half is the id the step before was fed
+                    meta.prev_ids = self._inflight["ids_dev"]
+            ids_used = ids
             with torch.inference_mode():
                 logits = self._pipeline_forward(meta, ids, meta.logits_indices)
         sp = [r.sampling_params for r in reqs]
@@ -633,6 +644,7 @@ class Engine:
             "rids": [r.rid for r in reqs],
             "reqs": list(reqs),
             "tokens_dev": tokens_dev,
+            "ids_dev": ids_used,
             "pinned": pinned,
             "event": event,
             "out_idx": slots_idx,
@@ -767,10 +779,14 @@ class Engine:
         # per-token Python loops per step — at 16 chunked-prefill steps that
         # was a visible TTFT slice
         bs = self.args.block_size
-        pos_parts, slot_parts, input_ids = [], [], []
+        pos_parts, slot_parts, input_ids, prev_ids = [], [], [], []
         block_tables, seq_lens, query_lens, logits_idx = [], [], [], []
         t = 0
         for c in chunks:
+            if self.uses_prev_tokens:
+                ids = c.req.prompt_token_ids
+                prev_ids.append(ids[c.start - 1] if c.start > 0 else -1)
+                prev_ids.extend(ids[c.start : c.start + c.num_tokens - 1])
             state = self.cache_manager.get(c.req.rid)
             pos = torch.arange(c.start, c.start + c.num_tokens, dtype=torch.int64)
             bt = torch.tensor(state.block_table, dtype=torch.int64)
@@ -799,6 +815,8 @@ class Engine:
             ) if self.linear_cache is not None else None,
             logits_indices=torch.tensor(logits_idx, dtype=torch.int64, device=dev),
             max_seq_len=max(seq_lens),
+            prev_ids=torch.tensor(prev_ids, dtype=torch.long, device=dev)
+            if self.uses_prev_tokens else None,
         )
         ids = torch.tensor(input_ids, dtype=torch.long, device=dev)
         return meta, ids
@@ -831,9 +849,17 @@ class Engine:
             ) if self.linear_cache is not None else None,
             logits_indices=torch.arange(len(reqs), dtype=torch.int64, device=dev),
             max_seq_len=max(seq_lens),
+            prev_ids=torch.tensor([r.decode_prev() for r in reqs],
+                                  dtype=torch.long, device=dev)
+            if self.uses_prev_tokens else None,
         )
         ids = torch.tensor(input_ids, dtype=torch.long, device=dev)
         return meta, ids
+
+    def _embed(self, input_ids: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
+        if self.uses_prev_tokens:
+            return self.model.embed(input_ids, meta.prev_ids).to(self.hidden_dtype)
+        return self.model.embed(input_ids).to(self.hidden_dtype)
 
     def _pipeline_forward(
         self, meta: ForwardMeta, input_ids: torch.Tensor, need_logits_at: torch.Tensor
@@ -844,7 +870,7 @@ class Engine:
         T = meta.num_tokens
         h = self.cfg.hidden_size
         if comm.is_first_stage:
-            hidden = self.model.embed(input_ids).to(self.hidden_dtype)
+            hidden = self._embed(input_ids, meta)
         else:
             hidden = comm.pp_recv((T, h), self.hidden_dtype, comm.pp_rank - 1)
         hidden = self.model(hidden, meta)
@@ -916,7 +942,7 @@ class Engine:
         if hidden_in is None and send_slot is None:
             return self._pipeline_forward(meta, input_ids, need)
         if comm.is_first_stage:
-            hidden = self.model.embed(input_ids).to(self.hidden_dtype)
+            hidden = self._embed(input_ids, meta)
         else:
             hidden = hidden_in
         hidden = self.model(hidden, meta)
@@ -936,7 +962,7 @@ class Engine:
         if self.graph_runner is None:
             meta, ids = self._build_decode_meta(reqs)
             if self.comm.is_first_stage:
-                hidden = self.model.embed(ids).to(self.hidden_dtype)
+                hidden = self._embed(ids, meta)
             else:
                 hidden = hidden_in
             hidden = self.model(hidden, meta)
@@ -963,7 +989,9 @@ class Engine:
         return self.graph_runner.run(input_ids, positions, slots, btabs, seq_lens,
                                      hidden_in=hidden_in,
                                      rids=[r.rid for r in reqs],
-                                     linear_slots=lin_slots)
+                                     linear_slots=lin_slots,
+                                     prev_ids=[r.decode_prev() for r in reqs]
+                                     if self.uses_prev_tokens else None)
 
     def _decode_one(self, reqs: List[InitialRequest]) -> Optional[torch.Tensor]:
         """Single-micro-batch decode with blocking PP transport."""

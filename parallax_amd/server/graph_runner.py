@@ -80,6 +80,10 @@ class DecodeGraphRunner:
 
         dev = device
         self.input_ids = torch.zeros(B, dtype=torch.long, device=dev)
+        # models whose embedding reads the (previous token, token) pair
+        self.uses_prev = bool(getattr(model, "uses_prev_tokens", False))
+        self.prev_ids = torch.full((B,), -1, dtype=torch.long, device=dev)
+        self.h_prev_ids = torch.full((B,), -1, dtype=torch.long, pin_memory=True)
         self.hidden_in = torch.zeros(B, hidden_size, dtype=dtype, device=dev)
         self.positions = torch.zeros(B, dtype=torch.int32, device=dev)
         self.slot_mapping = torch.full((B,), -1, dtype=torch.int64, device=dev)
@@ -132,12 +136,17 @@ class DecodeGraphRunner:
             linear_cache=self.linear_cache,
             linear_slots=self.linear_slots[:bucket]
             if self.linear_cache is not None else None,
+            prev_ids=self.prev_ids[:bucket] if self.uses_prev else None,
         )
 
     def _forward(self, bucket: int, ctx_bucket: Optional[int] = None) -> torch.Tensor:
         meta = self._meta(bucket, ctx_bucket)
         if self.is_first:
-            hidden = self.model.embed(self.input_ids[:bucket]).to(self.dtype)
+            if self.uses_prev:
+                hidden = self.model.embed(self.input_ids[:bucket],
+                                          meta.prev_ids).to(self.dtype)
+            else:
+                hidden = self.model.embed(self.input_ids[:bucket]).to(self.dtype)
         else:
             hidden = self.hidden_in[:bucket]
         hidden = self.model(hidden, meta)
@@ -151,6 +160,7 @@ class DecodeGraphRunner:
         # neutralize buffers: warmup/capture must not write into the live KV
         # cache (slot -1 = skip) or read past block-table row 0
         self.input_ids.zero_()
+        self.prev_ids.fill_(-1)
         self.positions.zero_()
         self.slot_mapping.fill_(-1)
         self.block_tables.zero_()
@@ -214,6 +224,7 @@ class DecodeGraphRunner:
         rids: Optional[List[str]] = None,
         linear_slots: Optional[List[int]] = None,
         input_ids_dev: Optional[torch.Tensor] = None,
+        prev_ids: Optional[List[int]] = None,
     ) -> torch.Tensor:
         """Returns logits[:B] (last stage) or hidden[:B] (other stages)."""
         B = len(seq_lens)
@@ -258,6 +269,16 @@ class DecodeGraphRunner:
         self._cached_btlens = btlens
         self._cached_tables = list(block_tables)
 
+        if self.uses_prev:
+            if input_ids_dev is None:
+                self.h_prev_ids[:B] = torch.tensor(prev_ids, dtype=torch.long)
+                self.h_prev_ids[B:bucket] = -1
+                self.prev_ids[:bucket].copy_(self.h_prev_ids[:bucket],
+                                             non_blocking=True)
+            else:
+                # pipelined decode feeds the same rows as the step before:
+                # what that step was fed is this step's predecessor
+                self.prev_ids[:B].copy_(self.input_ids[:B])
         if input_ids_dev is None:
             self.input_ids[:bucket].copy_(self.h_input_ids[:bucket],
                                           non_blocking=True)

@@ -128,6 +128,11 @@ class InitialRequest(Request):
             return self.prompt_token_ids[-1], self.prompt_len - 1
         return self.output_token_ids[-1], self.total_len - 1
 
+    def decode_prev(self) -> int:
+        """The token before the one decode_input() feeds (-1: there is none)."""
+        ids = self.prompt_token_ids if self.forced else self.all_token_ids()
+        return ids[-2] if len(ids) >= 2 else -1
+
     def commit_new_token(self, token_id: int) -> None:
         if self.first_token_time is None:
             self.first_token_time = time.monotonic()

@@ -54,6 +54,7 @@ mix_sources = [
     os.path.join(CSRC, "row_attention.hip"),
     os.path.join(CSRC, "row_attention_mfma.hip"),
     os.path.join(CSRC, "post_norm.hip"),
+    os.path.join(CSRC, "group_norm.hip"),
 ]
 
 wanted = [x for x in os.environ.get("PARALLAX_EXT", "_C,_mix").split(",") if x]
