@@ -310,6 +310,58 @@ def qwen3_moe_like_config(z: dict) -> dict:
     }
 
 
+# `--design-compare --design-pair pudizen`: a Pudizen stack (windowed
+# sigmoid-weighted attention, gated latent attention and softmax attention with
+# rotated values, each beside a squared-relu feed-forward that reads the same
+# grouped RMS norm; pair-hash embedding) beside a Qwen3-style dense stack
+# (grouped-query attention with q/k norm, the same windows on the same layers,
+# gated feed-forward) of EQUAL sizes.
+
+PUDIZEN_SIZES = {
+    "s": dict(width=1024, layers=8, heads=16, kv_heads=4, dim=64, ff=4096,
+              window=512, rank=128, vocab=32000),
+    "m": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=8192,
+              window=1024, rank=128, vocab=32000),
+}
+
+# layer kinds of the stack, repeated: window, latent, window, softmax
+_PUDIZEN_ORDER = ("attention_2", "latent_attention", "attention_2", "attention")
+
+
+def pudizen_config(z: dict) -> dict:
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    scale = z["dim"] ** -0.5
+    rot = {"dims": z["dim"] // 2, "base": 1e6}
+    layers = []
+    for i in range(z["layers"]):
+        kind = _PUDIZEN_ORDER[i % 4]
+        if kind == "latent_attention":
+            mx = {"heads": z["heads"], "dim": z["dim"], "vdim": z["dim"],
+                  "kv_rank": z["rank"], "scale": scale}
+        else:
+            mx = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"],
+                  "vdim": z["dim"], "scale": scale, "rot": dict(rot)}
+            if kind == "attention_2":
+                mx["mask"] = {"size": z["window"]}
+            else:
+                mx["rot"]["scaling"] = {"factor": 8.0, "low": 1.0, "high": 4.0,
+                                        "original": 8192}
+        layers.append({"type": kind, "mixer": mx, "mlp": mlp})
+    return {"architecture": "Pudizen", "layers": layers,
+            "norm": {"eps": 1e-6, "groups": 8},
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 100003,
+                                                   "mul_prev": 1000003,
+                                                   "mul_cur": 999983}},
+            "vocab": z["vocab"], "width": z["width"], "max_positions": 16384}
+
+
+def qwen3_like_pudizen_config(z: dict) -> dict:
+    cfg = qwen3_like_config(dict(z, pool=0))
+    cfg["layer_types"] = ["sliding_attention" if _PUDIZEN_ORDER[i % 4] == "attention_2"
+                          else "full_attention" for i in range(z["layers"])]
+    return cfg
+
+
 def design_compare(args) -> None:
     from parallax_amd.models.config import ModelConfig
     from parallax_amd.server.engine import Engine, EngineArgs
@@ -325,6 +377,10 @@ def design_compare(args) -> None:
             z = ZABUSUN_SIZES[size]
             pair = (("zabusun", zabusun_config(z)),
                     ("qwen3-moe-like", qwen3_moe_like_config(z)))
+        elif args.design_pair == "pudizen":
+            z = PUDIZEN_SIZES[size]
+            pair = (("pudizen", pudizen_config(z)),
+                    ("qwen3-like", qwen3_like_pudizen_config(z)))
         else:
             z = DESIGN_SIZES[size]
             pair = (("vurizen", vurizen_config(z)),
@@ -433,18 +489,20 @@ def main():
                          "throughput of a Vurizen stack beside a DeepSeek-V3-"
                          "style stack of equal sizes (one GPU, random weights)")
     ap.add_argument("--design-pair", default="vurizen",
-                    choices=["vurizen", "sogidra", "zabusun"],
+                    choices=["vurizen", "sogidra", "zabusun", "pudizen"],
                     help="which design --design-compare measures: vurizen "
                          "beside a DeepSeek-V3-style stack, sogidra beside "
-                         "a Qwen3-style dense stack, or zabusun beside a "
-                         "Qwen3-MoE-style stack")
+                         "a Qwen3-style dense stack, zabusun beside a "
+                         "Qwen3-MoE-style stack, or pudizen beside a "
+                         "Qwen3-style dense stack")
     ap.add_argument("--design-sizes", default="s,m",
                     help="comma list of " + ",".join(DESIGN_SIZES))
     ap.add_argument("--design-batch", type=int, default=8)
     ap.add_argument("--design-prompt", type=int, default=2048)
     ap.add_argument("--design-only", default="",
                     help="one design of the pair (vurizen | deepseek-like | "
-                         "sogidra | qwen3-like | zabusun | qwen3-moe-like; "
+                         "sogidra | qwen3-like | zabusun | qwen3-moe-like | "
+                         "pudizen; "
                          "default: both)")
     args = ap.parse_args()
     if args.design_compare:

@@ -160,12 +160,12 @@ class PudizenShardModel(nn.Module):
         self.groups = int(cfg.norm_groups)
         W = cfg.hidden_size
         if self.is_first:
-            ph = cfg.pair_hash
-            if ph is None:
-                raise ValueError("Pudizen needs embedding.bigram in its config")
+            # a config without a pair table: one bucket whose rows stay zero
+            ph = cfg.pair_hash or {"buckets": 1, "mul_prev": 0, "mul_cur": 0}
             self.embed_tokens = PairHashEmbedding(
                 cfg.vocab_size, W, ph["buckets"], ph["mul_prev"], ph["mul_cur"],
                 cfg.embed_scale)
+            self.embed_tokens.pair.data.zero_()
         self.layers = nn.ModuleList(
             PudizenLayer(cfg, cfg.layer_specs[g],
                          build_mixer(cfg.layer_specs[g]["type"],

@@ -307,27 +307,24 @@ class RotaryRowAttention(_RowAttentionBase):
         k, v = (parts[1], parts[2]) if self.owns_cache else (None, None)
         wq, wk, bias, (freq, vfreq), _ = self._constants(q.device)
         cache = meta.mla_cache.layer(self.cache_layer_idx)
+        # the tokens' cos/sin of the value rotation: the store turns the
+        # values by them, the attention kernel turns its results back
+        v_cs = torch.empty(q.shape[0], self.vdim, dtype=torch.float32,
+                           device=q.device) if vfreq is not None else None
         q32 = ops.qkv_store(
             q, k, v, meta.positions, meta.slot_mapping, cache, self.dim,
             self.eps if self.qk_norm_whole else None, 0.0, 0, q_weight=wq,
             k_weight=wk, rot_freq=freq, rot_mult=1.0, rot_dims=self.rot_dims,
             norm_whole=self.qk_norm_whole, rot_interleaved=self.rot_interleaved,
-            v_seg=self.vdim, v_rot_freq=vfreq if self.owns_cache else None)
-        o = ops.row_attention(
+            v_seg=self.vdim, v_rot_freq=vfreq, v_cs_out=v_cs)
+        return ops.row_attention(
             q32, cache, None, meta.block_tables, meta.token_seq(),
             meta.positions, self.heads, self.kv_heads, 1, self.dim, self.vdim,
-            self.window, 0, self.scale, 0.0, 0.0, None, 1.0,
-            torch.float32 if vfreq is not None else out_dtype,
+            self.window, 0, self.scale, 0.0, 0.0, None, 1.0, out_dtype,
             max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
-            head_bias=bias,
+            head_bias=bias, out_rot_cs=v_cs,
+            out_rot_interleaved=self.rot_interleaved,
         )
-        if vfreq is not None:
-            # the weighted sum of values turned by their positions, turned
-            # back by the query's position
-            o = ops.rotate_heads(o.view(-1, self.heads, self.vdim),
-                                 meta.positions, vfreq, self.rot_interleaved,
-                                 -1.0, out_dtype)
-        return o
 
     def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:
         parts = self.in_proj.split_output(self.in_proj(x))

@@ -295,6 +295,41 @@ __global__ __launch_bounds__(256) void rotate_heads_kernel(
   }
 }
 
+// the same with the tokens' (cos, sin) pairs given: table [T, D / 2][2]
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_heads_table_kernel(
+    T* __restrict__ out, const float* __restrict__ x,
+    const float* __restrict__ table, int H, int D, int inter, float sign) {
+  const int64_t t = blockIdx.x;
+  const int half = D / 2;
+  const float* cs = table + t * (int64_t)D;
+  const float* xr = x + t * (int64_t)H * D;
+  T* o = out + t * (int64_t)H * D;
+  const int n = H * half;
+  for (int idx = threadIdx.x; idx < n; idx += 256) {
+    const int h = idx / half, m = idx % half;
+    const int iu = h * D + (inter ? 2 * m : m);
+    const int iv = h * D + (inter ? 2 * m + 1 : m + half);
+    const float u = xr[iu], v = xr[iv];
+    const float c = cs[2 * m], sn = cs[2 * m + 1] * sign;
+    stf(o + iu, u * c - v * sn);
+    stf(o + iv, v * c + u * sn);
+  }
+}
+
+extern "C" void launch_rotate_heads_table(void* out, const float* x,
+                                          const float* table, int H, int D,
+                                          int inter, float sign, int T_,
+                                          int kind, hipStream_t stream) {
+  if (T_ == 0) return;
+  if (kind == 0)
+    hipLaunchKernelGGL((rotate_heads_table_kernel<bf16_t>), dim3(T_), dim3(256),
+                       0, stream, (bf16_t*)out, x, table, H, D, inter, sign);
+  else
+    hipLaunchKernelGGL((rotate_heads_table_kernel<float>), dim3(T_), dim3(256),
+                       0, stream, (float*)out, x, table, H, D, inter, sign);
+}
+
 extern "C" void launch_rotate_heads(void* out, const float* x, const float* freq,
                                     const int* positions, int H, int D,
                                     int inter, float sign, int T_, int kind,

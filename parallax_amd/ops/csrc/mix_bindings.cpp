@@ -41,23 +41,28 @@ void launch_qkv_store(float*, const void*, int64_t, const void*, int64_t,
                       const void*, int64_t, const int*, const int64_t*, void*,
                       int, int, int, int, float, float, int, const float*,
                       const float*, const float*, float, int, int, int,
-                      const float*, int, int, int, hipStream_t);
+                      const float*, int, float*, int, int, hipStream_t);
 void launch_pool_cache_update(const void*, float*, const int*, int, const int*,
                               const int*, const int64_t*, int, int, int, int,
                               int, int, hipStream_t);
 int row_attention_heads_per_group(int);
 int row_attention_prefill_supported(int, int);
+int row_attention_prefill_rotates(int, int);
+void launch_rotate_heads_table(void*, const float*, const float*, int, int,
+                               int, float, int, int, hipStream_t);
 void launch_row_attention_prefill(void*, float*, const float*, const void*,
                                   const float*, const int*, int, const int*,
                                   int, const int*, int, int, int, int, int, int,
                                   int, int, int, int, float, float, float,
                                   float, float, const float*, const void*,
-                                  int64_t, int, int, hipStream_t);
+                                  int64_t, int, const float*, int, int,
+                                  hipStream_t);
 void launch_row_attention(void*, float*, float*, const float*, const void*,
                           const float*, const int*, int, const int*, const int*,
                           int, int, int, int, int, int, int, int, int, int,
                           float, float, float, float, float, int, const float*,
-                          const void*, int64_t, int, int, hipStream_t);
+                          const void*, int64_t, int, const float*, int, int,
+                          hipStream_t);
 void launch_group_rmsnorm_add(float*, const void*, int64_t, const void*,
                               int64_t, const void*, float, void*, int, int,
                               int, int, hipStream_t);
@@ -388,7 +393,7 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                int64_t temp_every, torch::Tensor q_weight,
                torch::Tensor k_weight, torch::Tensor rot_freq, double rot_mult,
                int64_t rot_dims, bool norm_whole, bool rot_interleaved,
-               torch::Tensor v_rot_freq, int64_t v_seg) {
+               torch::Tensor v_rot_freq, int64_t v_seg, torch::Tensor v_cs_out) {
   const int kind = kind_of(q, "q");
   const bool has_qw = q_weight.numel() > 0, has_kw = k_weight.numel() > 0;
   const bool has_rot = rot_freq.numel() > 0 && rot_dims > 0;
@@ -407,11 +412,17 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                 k_weight.numel() == (norm_whole ? k.size(1) : seg),
                 "key norm weight width");
   }
+  // v_cs_out [T, v_seg] fp32: the tokens' (cos, sin) pairs of that rotation
+  const bool has_vcs = has_vrot && v_cs_out.numel() > 0;
   if (has_vrot) {
     CHECK_F32C(v_rot_freq);
-    TORCH_CHECK(v.dim() == 2 && v_seg > 0 && v_seg % 2 == 0 &&
-                v.size(1) % v_seg == 0 && v_rot_freq.numel() == v_seg / 2,
+    TORCH_CHECK(v_seg > 0 && v_seg % 2 == 0 && v_rot_freq.numel() == v_seg / 2 &&
+                (v.dim() != 2 || v.size(1) % v_seg == 0),
                 "rotated value segments");
+  }
+  if (has_vcs) {
+    CHECK_F32C(v_cs_out);
+    TORCH_CHECK(v_cs_out.numel() == q.size(0) * v_seg, "cos/sin table size");
   }
   if (has_rot) {
     CHECK_F32C(rot_freq);
@@ -460,7 +471,9 @@ void qkv_store(torch::Tensor q_out, torch::Tensor q, torch::Tensor k,
                    (float)rot_mult, has_rot ? (int)rot_dims : 0,
                    norm_whole ? 1 : 0, rot_interleaved ? 1 : 0,
                    has_vrot ? v_rot_freq.data_ptr<float>() : nullptr,
-                   has_vrot ? (int)v_seg : 0, T, kind, cur_stream());
+                   has_vrot ? (int)v_seg : 0,
+                   has_vcs ? v_cs_out.data_ptr<float>() : nullptr, T, kind,
+                   cur_stream());
 }
 
 // cache [blocks, block, E]; pool [blocks, per_page, E] fp32
@@ -502,7 +515,8 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
                    int64_t P, double scale, double softcap, double lam,
                    double norm_eps, double out_mult, int64_t max_keys,
                    torch::Tensor query_bounds, torch::Tensor head_bias,
-                   torch::Tensor gate, bool shared_kv) {
+                   torch::Tensor gate, bool shared_kv, torch::Tensor rot_cs,
+                   bool rot_interleaved) {
   const int kind = kind_of(cache, "cache");
   CHECK_F32C(q);
   // head_bias [H] fp32: sigmoid(score + head_bias[h]) weights, not normalised;
@@ -538,6 +552,16 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
               out.size(1) == H * dv);
   float* out32 = (kind == 0 && out.scalar_type() == torch::kFloat32)
                      ? out.data_ptr<float>() : nullptr;
+  // rot_cs [T, dv / 2][2] fp32 (cos, sin per token and pair): every head's
+  // result is turned back by its token's angles
+  const bool has_rot = rot_cs.numel() > 0;
+  if (has_rot) {
+    CHECK_F32C(rot_cs);
+    TORCH_CHECK(dv % 2 == 0 && rot_cs.numel() == (int64_t)T * dv,
+                "cos/sin table size");
+  }
+  const float* rot_p = has_rot ? rot_cs.data_ptr<float>() : nullptr;
+  const int rot_inter = rot_interleaved ? 1 : 0;
   TORCH_CHECK(window >= 0 && P >= 0);
   int per_page = 1;
   const bool has_pool = window > 0 && P > 0;
@@ -565,16 +589,32 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
     CHECK_I32(query_bounds);
     const int B = query_bounds.numel() - 1;
     TORCH_CHECK(B >= 1 && block_tables.size(0) >= B);
+    // a value width that does not fill its tile cannot pair halves in
+    // registers: fp32 results, then a pass of its own turns them
+    const bool turn_after =
+        has_rot && !row_attention_prefill_rotates((int)dv, rot_inter);
+    torch::Tensor tmp;
+    void* out_p = out.data_ptr();
+    float* out32_p = out32;
+    if (turn_after) {
+      tmp = torch::empty({(int64_t)T, H * dv}, q.options());
+      out_p = tmp.data_ptr();
+      out32_p = kind == 0 ? tmp.data_ptr<float>() : nullptr;
+    }
     launch_row_attention_prefill(
-        out.data_ptr(), out32, q.data_ptr<float>(), cache.data_ptr(),
+        out_p, out32_p, q.data_ptr<float>(), cache.data_ptr(),
         has_pool ? pool.data_ptr<float>() : nullptr,
         block_tables.data_ptr<int>(), (int)block_tables.stride(0),
         query_bounds.data_ptr<int>(), B, positions.data_ptr<int>(),
         (T + 31) / 32 + B, (int)H, (int)G, (int)M, (int)d, (int)dv,
         (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
         (float)scale, (float)softcap, (float)lam, (float)norm_eps,
-        (float)out_mult, bias_p, gate_p, gate_stride, vbase, kind,
-        cur_stream());
+        (float)out_mult, bias_p, gate_p, gate_stride, vbase,
+        turn_after ? nullptr : rot_p, rot_inter, kind, cur_stream());
+    if (turn_after)
+      launch_rotate_heads_table(out.data_ptr(), tmp.data_ptr<float>(), rot_p,
+                                (int)H, (int)dv, rot_inter, -1.0f, T,
+                                kind_of(out, "out"), cur_stream());
     return;
   }
   // shares of the key list per token: enough workgroups to fill the chip
@@ -605,8 +645,8 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
       positions.data_ptr<int>(), T, (int)H, (int)G, (int)M, (int)d, (int)dv,
       (int)cache.size(1), per_page, (int)window, has_pool ? (int)P : 0,
       (float)scale, (float)softcap, (float)lam, (float)norm_eps,
-      (float)out_mult, splits, bias_p, gate_p, gate_stride, vbase, kind,
-      cur_stream());
+      (float)out_mult, splits, bias_p, gate_p, gate_stride, vbase, rot_p,
+      rot_inter, kind, cur_stream());
 }
 
 // x [T, W] fp32 (updated in place when y1 is given); y1, y2 [T, W] of the

@@ -166,7 +166,7 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
     const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     const float* __restrict__ rot_freq, float rot_mult, int rot_dims,
     int staged, int vec, int whole, int inter,
-    const float* __restrict__ v_freq, int v_seg) {
+    const float* __restrict__ v_freq, int v_seg, float* __restrict__ v_cs_out) {
   __shared__ float red[8];
   const int64_t t = blockIdx.x;
   float temp = 1.0f;
@@ -197,6 +197,11 @@ __global__ __launch_bounds__(256) void qkv_store_kernel(
     }
   }
   __syncthreads();
+  // the token's (cos, sin) pairs of the value rotation, for the attention
+  // kernels that turn their results back
+  if (v_cs_out != nullptr)
+    for (int i = threadIdx.x; i < v_seg; i += 64 * RA_WAVES)
+      v_cs_out[t * v_seg + i] = v_cs[i];
   const bool full = NORM && whole;
   RaSegOps so{q_weight, rot_freq ? rot_cs : nullptr, rot_dims, inter != 0,
               full, 0.f};
@@ -238,14 +243,15 @@ extern "C" void launch_qkv_store(float* q_out, const void* q, int64_t q_stride,
                                  const float* q_weight, const float* k_weight,
                                  const float* rot_freq, float rot_mult,
                                  int rot_dims, int whole, int inter,
-                                 const float* v_freq, int v_seg, int T_,
-                                 int kind, hipStream_t stream) {
+                                 const float* v_freq, int v_seg,
+                                 float* v_cs_out, int T_, int kind,
+                                 hipStream_t stream) {
   if (T_ == 0) return;
 #define QS_ARGS(TT)                                                          \
   q_out, (const TT*)q, q_stride, (const TT*)k, k_stride, (const TT*)v,       \
       v_stride, positions, slots, (TT*)cache, wq, wk, wv, seg, eps,          \
       temp_coef, temp_every, q_weight, k_weight, rot_freq, rot_mult, rot_dims,  \
-      staged, vec, whole, inter, v_freq, v_seg
+      staged, vec, whole, inter, v_freq, v_seg, v_cs_out
   const bool norm = eps >= 0.f;
   // stage the token's queries and keys in LDS when they fit in 48 KB
   const int rot_floats = ((rot_freq ? rot_dims : 0) + 3) / 4 * 4 +
@@ -408,7 +414,8 @@ template <typename T, int M>
 DEVINL void ra_epilogue(T* __restrict__ dst, float* __restrict__ dst32,
                         const float* __restrict__ acc,
                         int acc_stride, const float* l, int dv, float lam,
-                        float norm_eps, float out_mult, float post) {
+                        float norm_eps, float out_mult, float post,
+                        const float* __restrict__ rcs, int rot_inter) {
   const int lane = threadIdx.x & 63;
   const float i0 = 1.0f / l[0];
   const float i1 = M == 2 ? lam / l[1] : 0.f;
@@ -421,6 +428,18 @@ DEVINL void ra_epilogue(T* __restrict__ dst, float* __restrict__ dst32,
     if (f < dv) {
       v = acc[f] * i0;
       if (M == 2) v -= acc[acc_stride + f] * i1;
+      if (rcs != nullptr) {
+        // rcs: the token's [dv / 2][2] cos, sin; the result turns BACK by its
+        // angle: pair (u, w) -> (u cos + w sin, w cos - u sin)
+        const int hv = dv >> 1;
+        const bool first = rot_inter ? !(f & 1) : f < hv;
+        const int fp = rot_inter ? (f ^ 1) : (first ? f + hv : f - hv);
+        const int m = rot_inter ? (f >> 1) : (first ? f : f - hv);
+        float w = acc[fp] * i0;
+        if (M == 2) w -= acc[acc_stride + fp] * i1;
+        const float cs = rcs[2 * m], sn = rcs[2 * m + 1];
+        v = first ? fmaf(w, sn, v * cs) : fmaf(-w, sn, v * cs);
+      }
     }
     o[c] = v;
     ss += v * v;
@@ -462,7 +481,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
     int G, int d, int dv, int block_size, int per_page, int window, int P,
     float scale, float softcap, float lam, float norm_eps, float out_mult,
     int splits, int FL, const float* __restrict__ head_bias,
-    const T* __restrict__ gate, int64_t gate_stride, int vbase) {
+    const T* __restrict__ gate, int64_t gate_stride, int vbase,
+    const float* __restrict__ rot_cs, int rot_inter) {
   constexpr int NQ = HB * M;
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -678,7 +698,8 @@ __global__ __launch_bounds__(256) void row_attention_kernel(
                         out32 ? out32 + (t * H + h) * (int64_t)dv : nullptr,
                         oacc + hh * M * dvp, dvp,
                         lg, dv, lam, norm_eps, out_mult,
-                        ra_gate<T>(gate, gate_stride, t, h));
+                        ra_gate<T>(gate, gate_stride, t, h),
+                        rot_cs ? rot_cs + t * dv : nullptr, rot_inter);
     } else {
 #pragma unroll
       for (int m = 0; m < M; ++m) {
@@ -701,7 +722,8 @@ __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
     T* __restrict__ out, float* __restrict__ out32,
     const float* __restrict__ part, int dv, int splits,
     float lam, float norm_eps, float out_mult, int H, int sig,
-    const T* __restrict__ gate, int64_t gate_stride) {
+    const T* __restrict__ gate, int64_t gate_stride,
+    const float* __restrict__ rot_cs, int rot_inter) {
   extern __shared__ float lds[];  // [M][dvp] sums | [M][64] weights
   const int64_t th = blockIdx.x;
   const int lane = threadIdx.x;
@@ -748,7 +770,8 @@ __global__ __launch_bounds__(64) void row_attention_reduce_kernel(
   ra_epilogue<T, M>(out + th * (int64_t)dv,
                     out32 ? out32 + th * (int64_t)dv : nullptr, lds, dvp, lg,
                     dv, lam, norm_eps,
-                    out_mult, ra_gate<T>(gate, gate_stride, th / H, (int)(th % H)));
+                    out_mult, ra_gate<T>(gate, gate_stride, th / H, (int)(th % H)),
+                    rot_cs ? rot_cs + (th / H) * dv : nullptr, rot_inter);
 }
 
 struct RaArgs {
@@ -769,6 +792,8 @@ struct RaArgs {
   const void* gate;
   int64_t gate_stride;
   int vbase;
+  const float* rot_cs;
+  int rot_inter;
   hipStream_t stream;
 };
 
@@ -794,7 +819,8 @@ static void launch_ra_hb(const RaArgs& a) {
                      a.positions, a.H, a.G, a.d, a.dv, a.block_size,          \
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,    \
                      a.norm_eps, a.out_mult, a.splits, FL, a.head_bias,       \
-                     (const T*)a.gate, a.gate_stride, a.vbase)
+                     (const T*)a.gate, a.gate_stride, a.vbase, a.rot_cs,      \
+                     a.rot_inter)
   const bool pooled = a.pool != nullptr && a.window > 0 && a.P > 0;
   if (vec) {
     if (pooled) RA_CALL(true, true);
@@ -810,7 +836,7 @@ static void launch_ra_hb(const RaArgs& a) {
                        a.stream, (T*)a.out, a.out32, a.part, a.dv, a.splits,
                        a.lam,
                        a.norm_eps, a.out_mult, a.H, a.head_bias != nullptr,
-                       (const T*)a.gate, a.gate_stride);
+                       (const T*)a.gate, a.gate_stride, a.rot_cs, a.rot_inter);
 }
 
 template <typename T, int M>
@@ -833,12 +859,12 @@ extern "C" void launch_row_attention(
     int block_size, int per_page, int window, int P, float scale, float softcap,
     float lam, float norm_eps, float out_mult, int splits,
     const float* head_bias, const void* gate, int64_t gate_stride, int vbase,
-    int kind, hipStream_t stream) {
+    const float* rot_cs, int rot_inter, int kind, hipStream_t stream) {
   if (T_ == 0) return;
   const RaArgs a{out, out32, part, q, cache, pool, block_tables, bt_stride, token_seq,
                  positions, T_, H, G, d, dv, block_size, per_page, window, P,
                  scale, softcap, lam, norm_eps, out_mult, splits, head_bias,
-                 gate, gate_stride, vbase, stream};
+                 gate, gate_stride, vbase, rot_cs, rot_inter, stream};
   if (kind == 0) {
     if (M == 1) launch_ra_m<bf16_t, 1>(a);
     else launch_ra_m<bf16_t, 2>(a);

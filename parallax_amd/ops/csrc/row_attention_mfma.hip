@@ -106,7 +106,8 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     int block_size, int per_page, int window, int P, float scale, float softcap,
     float lam, float norm_eps, float out_mult,
     const float* __restrict__ head_bias, const T* __restrict__ gate,
-    int64_t gate_stride, int vbase) {
+    int64_t gate_stride, int vbase, const float* __restrict__ rot_cs,
+    int rot_inter) {
   constexpr int DV = DVB * 32;
   constexpr int KS = D + RM_PAD, VS = DV + RM_PAD;
   constexpr int HW = 4 / M;  // heads per workgroup
@@ -424,6 +425,39 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[k][i] *= inv;
   }
+  if (rot_cs != nullptr) {
+    // the result turns BACK by the query's angle: rot_cs holds [dv / 2][2]
+    // cos, sin per token; pair (u, w) -> (u cos + w sin, w cos - u sin).
+    // Neighbouring pairs sit in one lane (i, i + 1); halves pair block k with
+    // block k + DVB / 2 when the value width fills the tile (the host sends
+    // other widths through a separate pass).
+    const float* rc = rot_cs + (int64_t)(t0 + min(col, nq - 1)) * dv;
+    if (rot_inter) {
+#pragma unroll
+      for (int k = 0; k < DVB; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+          if (f < dv) {
+            const float2 cs = *reinterpret_cast<const float2*>(rc + f);
+            const float u = acc[k][i], w = acc[k][i + 1];
+            acc[k][i] = fmaf(w, cs.y, u * cs.x);
+            acc[k][i + 1] = fmaf(-u, cs.y, w * cs.x);
+          }
+        }
+    } else {
+#pragma unroll
+      for (int k = 0; k < DVB / 2; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+          const float2 cs = *reinterpret_cast<const float2*>(rc + 2 * f);
+          const float u = acc[k][i], w = acc[k + DVB / 2][i];
+          acc[k][i] = fmaf(w, cs.y, u * cs.x);
+          acc[k + DVB / 2][i] = fmaf(-u, cs.y, w * cs.x);
+        }
+    }
+  }
   float r = 1.0f;
   if (norm_eps >= 0.f) {
     float ss = 0.f;
@@ -475,6 +509,8 @@ struct RmArgs {
   const void* gate;
   int64_t gate_stride;
   int vbase;
+  const float* rot_cs;
+  int rot_inter;
   hipStream_t stream;
 };
 
@@ -503,7 +539,7 @@ static void launch_rm_k(const RmArgs& a) {
                      a.cu, a.B, a.positions, a.H, a.G, a.d, a.dv, a.block_size,
                      a.per_page, a.window, a.P, a.scale, a.softcap, a.lam,
                      a.norm_eps, a.out_mult, a.head_bias, (const T*)a.gate,
-                     a.gate_stride, a.vbase);
+                     a.gate_stride, a.vbase, a.rot_cs, a.rot_inter);
 }
 
 // sigmoid weights come with one score map only
@@ -532,6 +568,13 @@ extern "C" int row_attention_prefill_supported(int d, int dv) {
   return d % 8 == 0 && dv % 8 == 0 && d <= 128 && dv <= 256;
 }
 
+// whether the matrix-core kernel can turn its results back in registers:
+// neighbouring pairs always; halves when the value width fills its tile
+extern "C" int row_attention_prefill_rotates(int dv, int inter) {
+  const int tile = dv <= 64 ? 64 : (dv <= 128 ? 128 : 256);
+  return inter || dv == tile;
+}
+
 // tiles: an upper bound on the number of 32-token tiles (ceil(T / 32) + B)
 extern "C" void launch_row_attention_prefill(
     void* out, float* out32, const float* q, const void* cache, const float* pool,
@@ -539,13 +582,13 @@ extern "C" void launch_row_attention_prefill(
     const int* positions, int tiles, int H, int G, int M, int d, int dv,
     int block_size, int per_page, int window, int P, float scale, float softcap,
     float lam, float norm_eps, float out_mult, const float* head_bias,
-    const void* gate, int64_t gate_stride, int vbase, int kind,
-    hipStream_t stream) {
+    const void* gate, int64_t gate_stride, int vbase, const float* rot_cs,
+    int rot_inter, int kind, hipStream_t stream) {
   if (tiles == 0) return;
   const RmArgs a{out, out32, q, cache, pool, block_tables, bt_stride, cu, B, positions,
                  tiles, H, G, d, dv, block_size, per_page, window, P, scale,
                  softcap, lam, norm_eps, out_mult, head_bias, gate, gate_stride,
-                 vbase, stream};
+                 vbase, rot_cs, rot_inter, stream};
   if (kind == 0) {
     if (M == 1) launch_rm_m<bf16_t, 1>(a);
     else launch_rm_m<bf16_t, 2>(a);

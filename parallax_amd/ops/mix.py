@@ -178,7 +178,7 @@ def sandwich_rmsnorm(x, y, w_branch, hist, n_hist, dwa, w_next, eps, offset,
 def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
               temp_coef, temp_every, q_weight=None, k_weight=None,
               rot_freq=None, rot_mult=1.0, rot_dims=0, norm_whole=False,
-              rot_interleaved=False, v_seg=0, v_rot_freq=None):
+              rot_interleaved=False, v_seg=0, v_rot_freq=None, v_cs_out=None):
     """Queries to fp32 (optionally RMS-normed per seg_dim-wide segment, with
     a weight [seg_dim] shared by the segments, or, with norm_whole, over the
     token's whole row with a weight as wide as the row; rotated by position
@@ -188,13 +188,16 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
     (normed, weighted and rotated alike) and values scattered as one row
     [keys | values] per token into the paged cache. v_rot_freq [v_seg / 2]:
     every v_seg-wide segment of the values is rotated over its whole width
-    (same pairing) before it is stored. v None: values = the keys before the
-    norm. k None: no store."""
+    (same pairing) before it is stored, and v_cs_out [T, v_seg] fp32 receives
+    the tokens' (cos, sin) pairs of that rotation (for row_attention's
+    out_rot_cs). v None: values = the keys before the norm. k None: no
+    store."""
     if not q.is_cuda:
         return ref.qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim,
                              norm_eps, temp_coef, temp_every, q_weight,
                              k_weight, rot_freq, rot_mult, rot_dims,
-                             norm_whole, rot_interleaved, v_seg, v_rot_freq)
+                             norm_whole, rot_interleaved, v_seg, v_rot_freq,
+                             v_cs_out)
     out = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     e = _empty(q)
     ef = _empty(q, torch.float32)
@@ -209,6 +212,7 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
         int(rot_dims) if rot_freq is not None else 0,
         bool(norm_whole), bool(rot_interleaved),
         v_rot_freq if v_rot_freq is not None else ef, int(v_seg),
+        v_cs_out if v_cs_out is not None else ef,
     )
     return out
 
@@ -231,7 +235,7 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0,
                   query_bounds=None, head_bias=None, gate=None,
-                  shared_kv=False):
+                  shared_kv=False, out_rot_cs=None, out_rot_interleaved=False):
     """Attention of fp32 queries over paged cache rows [keys | values] with
     grouped heads: full causal (window 0) or a sliding window with pooled
     blocks beyond it, optional tanh soft cap, one or two score maps per head
@@ -245,14 +249,17 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
     tokens of sequence b are query_bounds[b] .. query_bounds[b+1], at
     consecutive positions) lets the GPU path tile 32 tokens per workgroup on
     the fp32 matrix cores. shared_kv: a cache row holds the keys only and a
-    kv head's values are its keys (one map, vdim == dim). Returns [T, heads *
+    kv head's values are its keys (one map, vdim == dim). out_rot_cs [T,
+    vdim] fp32 ((cos, sin) per token and pair, as qkv_store's v_cs_out gives
+    them): every head's result is turned back by its token's angles over the
+    whole value width, in the epilogue of the attention kernel. Returns [T, heads *
     vdim] of out_dtype (the cache's type, or float32)."""
     if not q.is_cuda:
         return ref.row_attention(q, cache, pool, block_tables, token_seq,
                                  positions, heads, kv_heads, maps, dim, vdim,
                                  window, pool_tokens, scale, softcap, lam,
                                  norm_eps, out_mult, out_dtype, head_bias, gate,
-                                 shared_kv)
+                                 shared_kv, out_rot_cs, out_rot_interleaved)
     if head_bias is not None and maps != 1:
         raise ValueError("sigmoid key weights take one score map per head")
     out = torch.empty(q.shape[0], heads * vdim, dtype=out_dtype, device=q.device)
@@ -271,6 +278,7 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         else _empty(positions),
         head_bias if head_bias is not None else ef,
         gate if gate is not None else ef, bool(shared_kv),
+        out_rot_cs if out_rot_cs is not None else ef, bool(out_rot_interleaved),
     )
     return out
 

@@ -716,7 +716,7 @@ def _segment_rotate(x, seg, positions, freq, mult, rot_dims, interleaved=False):
 def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
               temp_coef, temp_every, q_weight=None, k_weight=None,
               rot_freq=None, rot_mult=1.0, rot_dims=0, norm_whole=False,
-              rot_interleaved=False, v_seg=0, v_rot_freq=None):
+              rot_interleaved=False, v_seg=0, v_rot_freq=None, v_cs_out=None):
     """Queries to fp32 (each seg_dim-wide segment divided by its RMS when
     norm_eps is given, times q_weight [seg_dim] when given; with norm_whole
     the RMS runs over the token's WHOLE query row and q_weight has the row's
@@ -728,7 +728,8 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
     k_weight and rotated alike) and values into one cache row [keys | values]
     per token. v_rot_freq [v_seg / 2] given: every v_seg-wide segment of the
     values is rotated by position over its whole width (same pairing, angles
-    pos * v_rot_freq[m]) before it is stored. v None: the values are the keys
+    pos * v_rot_freq[m]) before it is stored; v_cs_out [T, v_seg] fp32 then
+    receives every token's (cos, sin) pairs of that rotation. v None: the values are the keys
     as they came in, before the norm. k None: nothing is stored (the layer
     reads another layer's rows). Slot -1 skips the token."""
 
@@ -746,6 +747,10 @@ def qkv_store(q, k, v, positions, slot_mapping, cache, seg_dim, norm_eps,
         return x
 
     qf = prepare(q.float(), q_weight)
+    if v_rot_freq is not None and v_cs_out is not None:
+        ang = positions.float().unsqueeze(-1) * v_rot_freq.float()
+        v_cs_out.copy_(torch.stack([torch.cos(ang), torch.sin(ang)], -1)
+                       .reshape(v_cs_out.shape))
     if temp_every > 0:
         p = positions.float()
         temp = 1.0 + temp_coef * torch.log(torch.floor((p + 1.0) / temp_every) + 1.0)
@@ -801,7 +806,8 @@ def pool_cache_update(cache, pool, block_tables, token_seq, positions,
 def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, head_bias=None,
-                  gate=None, shared_kv=False):
+                  gate=None, shared_kv=False, out_rot_cs=None,
+                  out_rot_interleaved=False):
     """Attention over cache rows [keys (kv_heads x maps x dim) |
     values (kv_heads x vdim)]; shared_kv: a row holds the keys only and a kv
     head's values ARE its keys (vdim == dim, one map). q [T, heads * maps * dim] fp32. window 0: every
@@ -814,6 +820,10 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
     head_bias [heads] given: no softmax; a visible key weighs sigmoid(s +
     head_bias[h]) and the weights are not normalised over the keys. gate
     [T, heads] given: head h's result is multiplied by sigmoid(gate[t, h]).
+    out_rot_cs [T, vdim / 2, 2] (cos, sin per token and pair) given: every
+    head's result is turned BACK by its token's angles over the whole value
+    width (pair m = dimensions m, m + vdim / 2, or 2m, 2m + 1 when
+    out_rot_interleaved): (u, w) -> (u cos + w sin, w cos - u sin).
     Returns [T, heads * vdim] in out_dtype."""
     T = q.shape[0]
     bs = cache.shape[1]
@@ -851,6 +861,18 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         if gate is not None:
             o = o * torch.sigmoid(gate[t].float()).view(G, rep, 1)
         out[t] = o.reshape(H, vdim)
+    if out_rot_cs is not None:
+        cs = out_rot_cs.view(T, 1, vdim // 2, 2).float()
+        c, sn = cs[..., 0], cs[..., 1]
+        if out_rot_interleaved:
+            u, w = out[..., 0::2].clone(), out[..., 1::2].clone()
+            out[..., 0::2] = u * c + w * sn
+            out[..., 1::2] = w * c - u * sn
+        else:
+            hv = vdim // 2
+            u, w = out[..., :hv].clone(), out[..., hv:].clone()
+            out[..., :hv] = u * c + w * sn
+            out[..., hv:] = w * c - u * sn
     return out.view(T, H * vdim).to(out_dtype)
 
 

@@ -130,8 +130,12 @@ class InitialRequest(Request):
 
     def decode_prev(self) -> int:
         """The token before the one decode_input() feeds (-1: there is none)."""
-        ids = self.prompt_token_ids if self.forced else self.all_token_ids()
-        return ids[-2] if len(ids) >= 2 else -1
+        if self.forced or not self.output_token_ids:
+            ids = self.prompt_token_ids
+            return ids[-2] if len(ids) >= 2 else -1
+        if len(self.output_token_ids) >= 2:
+            return self.output_token_ids[-2]
+        return self.prompt_token_ids[-1] if self.prompt_token_ids else -1
 
     def commit_new_token(self, token_id: int) -> None:
         if self.first_token_time is None:
