@@ -104,6 +104,8 @@ class GatedLatentAttention(nn.Module):
     caller merges the input projections (widths `proj_sizes`: queries, latent,
     gate pre-activations) with others of the same input and calls mix()."""
 
+    VALUE_COLS = 256   # value columns a head sums in one attention call
+
     def __init__(self, hidden_size: int, heads: int, dim: int, value_dim: int,
                  rank: int, scale: float, norm_eps: float, cache_layer_idx: int,
                  own_proj: bool = True):
@@ -140,14 +142,22 @@ class GatedLatentAttention(nn.Module):
         ops.latent_kv_store(dkv, self.latent_norm, self.eps, no_freq, 1.0, 0,
                             meta.positions, meta.slot_mapping, cache, self.rank)
         q_lat = torch.einsum("thd,hdr->thr", q.view(T, H, self.dim).float(), w_uk)
-        o_lat = ops.row_attention(
-            q_lat.reshape(T, H * self.rank), cache, None, meta.block_tables,
-            meta.token_seq(), meta.positions, H, 1, 1, self.rank, self.rank,
-            0, 0, self.scale, 0.0, 0.0, None, 1.0, torch.float32,
-            max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
-            gate=gate, shared_kv=True,
-        )
-        attn = torch.einsum("thr,hvr->thv", o_lat.view(T, H, self.rank), w_uv)
+        q_lat = q_lat.reshape(T, H * self.rank)
+        # the attention kernels sum at most VALUE_COLS value columns per
+        # head: a wider latent is summed in column shares (the scores are
+        # worked out again for every share)
+        shares = []
+        for c0 in range(0, self.rank, self.VALUE_COLS):
+            cols = min(self.VALUE_COLS, self.rank - c0)
+            shares.append(ops.row_attention(
+                q_lat, cache, None, meta.block_tables, meta.token_seq(),
+                meta.positions, H, 1, 1, self.rank, cols, 0, 0, self.scale,
+                0.0, 0.0, None, 1.0, torch.float32,
+                max_seq_len=meta.max_seq_len, query_bounds=meta.query_bounds(),
+                gate=gate, shared_kv=True, value_col=c0,
+            ).view(T, H, cols))
+        o_lat = shares[0] if len(shares) == 1 else torch.cat(shares, dim=-1)
+        attn = torch.einsum("thr,hvr->thv", o_lat, w_uv)
         return attn.to(out_dtype).reshape(T, H * self.vdim)
 
     def forward(self, x: torch.Tensor, meta: ForwardMeta) -> torch.Tensor:

@@ -515,7 +515,7 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
                    int64_t P, double scale, double softcap, double lam,
                    double norm_eps, double out_mult, int64_t max_keys,
                    torch::Tensor query_bounds, torch::Tensor head_bias,
-                   torch::Tensor gate, bool shared_kv, torch::Tensor rot_cs,
+                   torch::Tensor gate, int64_t value_col, torch::Tensor rot_cs,
                    bool rot_interleaved) {
   const int kind = kind_of(cache, "cache");
   CHECK_F32C(q);
@@ -540,10 +540,13 @@ void row_attention(torch::Tensor out, torch::Tensor q, torch::Tensor cache,
   TORCH_CHECK(dv <= 256, "value width above 256 is not supported");
   TORCH_CHECK(d <= 1024, "key width above 1024 is not supported");
   TORCH_CHECK(q.size(1) == H * M * d, "query width");
-  // shared_kv: a row holds the keys only and a kv head's values are its keys
-  if (shared_kv) TORCH_CHECK(M == 1 && d == dv, "shared keys and values");
-  const int vbase = shared_kv ? 0 : (int)(G * M * d);
-  const int E = vbase + G * dv;
+  // value_col < 0: a row is [keys | values]. value_col >= 0: a row holds the
+  // keys only and the values are its columns from value_col on (0 with dv ==
+  // d: the values ARE the keys; other columns: a share of a wide latent row)
+  if (value_col >= 0)
+    TORCH_CHECK(M == 1 && G == 1 && value_col + dv <= d, "shared keys and values");
+  const int vbase = value_col >= 0 ? (int)value_col : (int)(G * M * d);
+  const int E = std::max<int>((int)(G * M * d), vbase + (int)(G * dv));
   TORCH_CHECK(cache.size(2) == E, "cache row width");
   // the result has the cache's type, or fp32
   TORCH_CHECK(out.is_cuda() && (out.scalar_type() == cache.scalar_type() ||

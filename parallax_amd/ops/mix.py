@@ -235,7 +235,8 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, max_seq_len=0,
                   query_bounds=None, head_bias=None, gate=None,
-                  shared_kv=False, out_rot_cs=None, out_rot_interleaved=False):
+                  shared_kv=False, out_rot_cs=None, out_rot_interleaved=False,
+                  value_col=0):
     """Attention of fp32 queries over paged cache rows [keys | values] with
     grouped heads: full causal (window 0) or a sliding window with pooled
     blocks beyond it, optional tanh soft cap, one or two score maps per head
@@ -248,8 +249,9 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
     long key ranges over workgroups. query_bounds [B+1] int32 (prompt portions:
     tokens of sequence b are query_bounds[b] .. query_bounds[b+1], at
     consecutive positions) lets the GPU path tile 32 tokens per workgroup on
-    the fp32 matrix cores. shared_kv: a cache row holds the keys only and a
-    kv head's values are its keys (one map, vdim == dim). out_rot_cs [T,
+    the fp32 matrix cores. shared_kv: a cache row holds the keys only (one kv
+    head, one map) and the values are its columns value_col .. value_col +
+    vdim (vdim == dim: the values are the keys). out_rot_cs [T,
     vdim] fp32 ((cos, sin) per token and pair, as qkv_store's v_cs_out gives
     them): every head's result is turned back by its token's angles over the
     whole value width, in the epilogue of the attention kernel. Returns [T, heads *
@@ -259,7 +261,8 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                                  positions, heads, kv_heads, maps, dim, vdim,
                                  window, pool_tokens, scale, softcap, lam,
                                  norm_eps, out_mult, out_dtype, head_bias, gate,
-                                 shared_kv, out_rot_cs, out_rot_interleaved)
+                                 shared_kv, out_rot_cs, out_rot_interleaved,
+                                 value_col)
     if head_bias is not None and maps != 1:
         raise ValueError("sigmoid key weights take one score map per head")
     out = torch.empty(q.shape[0], heads * vdim, dtype=out_dtype, device=q.device)
@@ -277,7 +280,7 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
         query_bounds if query_bounds is not None and token_seq is not None
         else _empty(positions),
         head_bias if head_bias is not None else ef,
-        gate if gate is not None else ef, bool(shared_kv),
+        gate if gate is not None else ef, int(value_col) if shared_kv else -1,
         out_rot_cs if out_rot_cs is not None else ef, bool(out_rot_interleaved),
     )
     return out

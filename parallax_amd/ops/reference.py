@@ -807,10 +807,11 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
                   kv_heads, maps, dim, vdim, window, pool_tokens, scale,
                   softcap, lam, norm_eps, out_mult, out_dtype, head_bias=None,
                   gate=None, shared_kv=False, out_rot_cs=None,
-                  out_rot_interleaved=False):
+                  out_rot_interleaved=False, value_col=0):
     """Attention over cache rows [keys (kv_heads x maps x dim) |
-    values (kv_heads x vdim)]; shared_kv: a row holds the keys only and a kv
-    head's values ARE its keys (vdim == dim, one map). q [T, heads * maps * dim] fp32. window 0: every
+    values (kv_heads x vdim)]; shared_kv: a row holds the keys only (one kv
+    head, one map) and the values are its columns value_col .. value_col +
+    vdim (vdim == dim: the values ARE the keys). q [T, heads * maps * dim] fp32. window 0: every
     key up to the token's position; window > 0: keys j with 0 <= pos - j <
     window plus, when pool_tokens > 0, the pooled row of every block of
     pool_tokens positions that ends at or before pos - window, in the same
@@ -846,7 +847,8 @@ def row_attention(q, cache, pool, block_tables, token_seq, positions, heads,
             per_page = pool.shape[1]
             rows = torch.cat([pool[bt[b // per_page], b % per_page], rows], 0)
         k = rows[:, :wk].view(-1, G, M, dim)
-        v = rows[:, (0 if shared_kv else wk):].view(-1, G, vdim)
+        v = (rows[:, value_col:value_col + vdim] if shared_kv
+             else rows[:, wk:]).reshape(-1, G, vdim)
         s = torch.einsum("grmd,ngmd->grmn", qv[t], k) * scale
         if softcap > 0:
             s = softcap * torch.tanh(s / softcap)

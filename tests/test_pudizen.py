@@ -190,6 +190,19 @@ def test_each_mixer_alone_portions_and_pages(li):
     torch.testing.assert_close(got.double(), want, rtol=2e-4, atol=2e-4)
 
 
+def test_a_latent_wider_than_one_share_of_value_columns():
+    """The attention kernels sum a bounded number of value columns per head;
+    a wider latent is summed in shares of its columns."""
+    spec = U.latent_layer(3, 8, 12, 300, 0.3, None)
+    w = oracle.random_weights(U.small_config([spec]), seed=33)
+    layer = _one_layer(spec, w)
+    assert layer.mixer.rank > layer.mixer.VALUE_COLS
+    h = torch.randn(40, WIDTH, generator=torch.Generator().manual_seed(8))
+    want = oracle.latent_attention(h.double(), w, "l0.mix.", spec["mixer"], EPS)
+    got = _run_cut(layer, h, [9, 1, 1, 29], 8, [3, 1, 4, 0, 2], _cache_for(spec, 8, 5))
+    torch.testing.assert_close(got.double(), want, rtol=2e-4, atol=2e-4)
+
+
 def test_softmax_attention_with_a_window_too():
     """The window is a switch of the mixer class, not of a layer type."""
     spec = U.softmax_layer(4, 2, 8, 12, 0.4, U.rot(4, 50.0, None), None, window=7)

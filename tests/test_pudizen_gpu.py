@@ -127,13 +127,15 @@ def test_sizes_outside_the_tuned_paths(tmp_path, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_long_contexts_and_wide_heads(tmp_path, dtype):
     """Key and value widths on the matrix-core tiles and off them, head groups
-    of 8, 3 and 5, a latent of 96 under 8 heads, contexts of many pages and a
+    of 8, 3 and 5, a latent of 96 under 8 heads and one of 320 (summed in two
+    shares of its columns) under 2, contexts of many pages and a
     window of several: long portions take the tiled kernel, single tokens the
     per-token one with split key lists, and both agree with the reference."""
     layers = [U.softmax_layer(8, 2, 96, 80, 0.1, U.rot(32, 40000.0), U.dense(96)),
               U.window_layer(3, 1, 128, 256, 0.08, 200, U.rot(128, 1000.0, None), None),
               U.latent_layer(8, 48, 32, 96, 0.15, U.dense(128)),
-              U.softmax_layer(5, 5, 104, 40, 0.1, U.rot(10), U.dense(128))]
+              U.softmax_layer(5, 5, 104, 40, 0.1, U.rot(10), U.dense(128)),
+              U.latent_layer(2, 16, 24, 320, 0.2, None)]
     cfg = U.small_config(layers, width=128, vocab=211, groups=8)
     w = oracle.random_weights(cfg, seed=23)
     path = U.write_checkpoint(str(tmp_path), cfg, w)

@@ -148,7 +148,7 @@ def test_store_and_attention(dt, H, G, d, dv, rot, inter, whole, vrot, win, sig)
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("H,r", [(8, 64), (3, 24), (5, 20), (2, 256)])
+@pytest.mark.parametrize("H,r", [(8, 64), (3, 24), (5, 20), (2, 256), (2, 320)])
 def test_rows_whose_values_are_their_keys(dt, H, r):
     g = torch.Generator().manual_seed(H + r)
     bs = 16
@@ -169,9 +169,28 @@ def test_rows_whose_values_are_their_keys(dt, H, r):
     want = ref.row_attention(ql, cc, None, bt, seq, pos, H, 1, 1, r, r, 0, 0, 0.2, 0.0, 0.0,
                              None, 1.0, torch.float32, None, gate, True)
     for tiled in (True, False):
+        if r > 256:      # more value columns than a head sums in one call
+            with pytest.raises(RuntimeError):
+                ops.row_attention(ql.to(DEV), cc.to(DEV), None, bt.to(DEV), seq.to(DEV),
+                                  pos.to(DEV), H, 1, 1, r, r, 0, 0, 0.2, 0.0, 0.0, None, 1.0,
+                                  torch.float32, gate=gate.to(DEV), shared_kv=True)
+            break
         got = ops.row_attention(ql.to(DEV), cc.to(DEV), None, bt.to(DEV), seq.to(DEV),
                                 pos.to(DEV), H, 1, 1, r, r, 0, 0, 0.2, 0.0, 0.0, None, 1.0,
                                 torch.float32, max_seq_len=70,
                                 query_bounds=bounds.to(DEV) if tiled else None,
                                 gate=gate.to(DEV), shared_kv=True)
         assert close(got, want, 2e-5), tiled
+    # a share of the row's columns as values
+    if r >= 24:
+        c0, cols = (8, r - 16) if r <= 256 else (256, r - 256)
+        want = ref.row_attention(ql, cc, None, bt, seq, pos, H, 1, 1, r, cols, 0, 0, 0.2, 0.0,
+                                 0.0, None, 1.0, torch.float32, None, gate, True, None, False,
+                                 c0)
+        for tiled in (True, False):
+            got = ops.row_attention(ql.to(DEV), cc.to(DEV), None, bt.to(DEV), seq.to(DEV),
+                                    pos.to(DEV), H, 1, 1, r, cols, 0, 0, 0.2, 0.0, 0.0, None,
+                                    1.0, torch.float32, max_seq_len=70,
+                                    query_bounds=bounds.to(DEV) if tiled else None,
+                                    gate=gate.to(DEV), shared_kv=True, value_col=c0)
+            assert close(got, want, 2e-5), (tiled, "share")
