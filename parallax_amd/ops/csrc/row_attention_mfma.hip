@@ -31,6 +31,9 @@
 // SIG instantiations replace the softmax by sigmoid(score + head_bias[h])
 // weights that are not normalised over the keys: no running maximum, no
 // rescaling of the accumulators, masked keys weigh 0.
+#include <cstdlib>
+#include <type_traits>
+
 #include "seq_common.h"
 
 typedef float f32x16v __attribute__((ext_vector_type(16)));
@@ -492,6 +495,326 @@ __global__ __launch_bounds__(256, 2) void row_attention_prefill_kernel(
     }
 }
 
+// ---- bf16 cache rows: the same products on the bf16 matrix cores, exactly ----
+//
+// With bf16 cache rows a key or value element IS a bf16 number, and an fp32
+// query element (or key weight) x is exactly the sum of three bf16 numbers:
+// its top 8 mantissa bits, the top 8 of what is left, and the rest. So
+//     q . k = q_hi . k + q_mid . k + q_lo . k
+// holds term by term in fp32 (a product of two bf16 numbers is exact in fp32,
+// the sums run in the fp32 accumulator), and likewise sum_j p_j v_j with p
+// split. Three v_mfma_f32_32x32x16_bf16 per 16 contracted elements do the
+// work of eight v_mfma_f32_32x32x2_f32 at one sixteenth of their cost each.
+// Same tiling, masks, softmax, accumulator layout and epilogue as the kernel
+// above; one score map, no pooled rows. K rows go to LDS as they are (no
+// conversion), V goes in transposed ([feature][key]) so that a lane reads the
+// 8 keys of its slots in two 8-byte pieces.
+//
+// Operand slots: lane (col = lane % 32, half = lane / 32) supplies 8 of the
+// 16 contracted elements of an instruction. Both operands put the SAME
+// element into the same slot, which is all the instruction asks for:
+//   scores, step s:  slot e <-> feature 16 s + 8 half + e
+//   values, step s:  slot e <-> key 16 s + 4 half + e (e < 4),
+//                               key 16 s + 8 + 4 half + e - 4 (e >= 4)
+// (the keys whose weights the lane's score registers 8 s .. 8 s + 7 hold).
+
+DEVINL void rb_split3(float x, short& hi, short& mid, short& lo) {
+  const uint32_t b0 = __float_as_uint(x) & 0xffff0000u;
+  const float r1 = x - __uint_as_float(b0);          // exact
+  const uint32_t b1 = __float_as_uint(r1) & 0xffff0000u;
+  const float r2 = r1 - __uint_as_float(b1);         // exact, at most 8 bits left
+  hi = (short)(b0 >> 16);
+  mid = (short)(b1 >> 16);
+  lo = (short)(__float_as_uint(r2) >> 16);
+}
+
+#define RB_KPAD 8   // bf16 elements of padding per K row (16 bytes)
+#define RB_VS 36    // bf16 elements per transposed V row: 32 keys + 4 (72 bytes)
+
+template <int D, int DVB, bool SIG>
+__global__ __launch_bounds__(256, 2) void row_attention_prefill_bf16_kernel(
+    bf16_t* __restrict__ out, float* __restrict__ out32, const float* __restrict__ q,
+    const bf16_t* __restrict__ cache, const int* __restrict__ block_tables,
+    int bt_stride, const int* __restrict__ cu, int B,
+    const int* __restrict__ positions, int H, int G, int d, int dv,
+    int block_size, int window, float scale, float softcap, float norm_eps,
+    float out_mult, const float* __restrict__ head_bias,
+    const bf16_t* __restrict__ gate, int64_t gate_stride, int vbase,
+    const float* __restrict__ rot_cs, int rot_inter) {
+  constexpr int DV = DVB * 32;
+  constexpr int KS = D + RB_KPAD;
+  constexpr int HW = 4;  // heads per workgroup
+  extern __shared__ float lds[];
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(lds);   // [32][KS]
+  bf16_t* Vt = Ks + RM_K * KS;                    // [DV][RB_VS]
+
+  int tile = gridDim.x - 1 - blockIdx.x, b = 0;
+  for (; b < B; ++b) {
+    const int nt = (cu[b + 1] - cu[b] + RM_Q - 1) / RM_Q;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (b == B) return;
+  const int t0 = cu[b] + tile * RM_Q;
+  const int nq = min(RM_Q, cu[b + 1] - t0);
+  const int p0 = positions[t0], p_last = p0 + nq - 1;
+  const int* bt = block_tables + (int64_t)b * bt_stride;
+
+  const int rep = H / G;
+  const int nhw = (rep + HW - 1) / HW;
+  const int g = blockIdx.y / nhw;
+  const int r0 = (blockIdx.y % nhw) * HW;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int half = lane >> 5, col = lane & 31;
+  const bool stream_on = r0 + wave < rep;
+  const int h = g * rep + min(r0 + wave, rep - 1);
+  const int wkeys = G * d;
+  const int E = max(wkeys, vbase + G * dv);
+  const int kcol = g * d, vcol = vbase + g * dv;
+
+  const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int nk = p_last - lo + 1;
+
+  // the lane's query (column col) in three bf16 parts, slot order
+  bf16x8v qh[D / 16], qm[D / 16], ql[D / 16];
+  {
+    const bool on = stream_on && col < nq;
+    const float* src = q + ((int64_t)(t0 + min(col, nq - 1)) * H + h) * d;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int f = 16 * s + 8 * half + e;
+        const float x = (on && f < d) ? src[f] : 0.f;
+        short a, m, l;
+        rb_split3(x, a, m, l);
+        qh[s][e] = a;
+        qm[s][e] = m;
+        ql[s][e] = l;
+      }
+  }
+  const int pq = p0 + col;
+  const bool qvalid = col < nq;
+
+  f32x16v acc[DVB];
+#pragma unroll
+  for (int k = 0; k < DVB; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[k][i] = 0.f;
+  float mx = -INFINITY, l = 0.f;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  const float hbias = SIG ? head_bias[h] : 0.f;
+
+  // staging role: 8 threads per key row, 8 elements each at a time
+  const int srow = threadIdx.x >> 3, ssub = threadIdx.x & 7;
+  constexpr int KC = D / 64, VC = (DV + 63) / 64;
+  int4 kraw[KC], vraw[VC];
+  auto fetch = [&](int u0) {
+    const int u = u0 + srow;
+    const bool on = u < nk;
+    int64_t off = 0;
+    if (on) {
+      const int j = lo + u;
+      off = ((int64_t)bt[j / block_size] * block_size + j % block_size) * E;
+    }
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int f = ssub * 8 + 64 * c;
+      kraw[c] = (on && f < d) ? *reinterpret_cast<const int4*>(cache + off + kcol + f)
+                              : make_int4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int f = ssub * 8 + 64 * c;
+      vraw[c] = (on && f < dv) ? *reinterpret_cast<const int4*>(cache + off + vcol + f)
+                               : make_int4(0, 0, 0, 0);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int c = 0; c < KC; ++c)
+      *reinterpret_cast<int4*>(Ks + srow * KS + ssub * 8 + 64 * c) = kraw[c];
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int f = ssub * 8 + 64 * c;
+      if (f < DV) {
+        const uint32_t w[4] = {(uint32_t)vraw[c].x, (uint32_t)vraw[c].y,
+                               (uint32_t)vraw[c].z, (uint32_t)vraw[c].w};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          Vt[(f + e) * RB_VS + srow] =
+              (bf16_t)((e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu));
+      }
+    }
+  };
+
+  bool fetched = false;
+  for (int u0 = 0; u0 < nk; u0 += RM_K) {
+    __syncthreads();  // the previous step's reads are done
+    if (!fetched) fetch(u0);
+    stash();
+    __syncthreads();
+    fetched = u0 + RM_K < nk;
+    if (fetched) fetch(u0 + RM_K);
+
+    // ---- S^T = K_tile . Q^T, three parts of q ------------------------------------
+    f32x16v S;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) S[i] = 0.f;
+    {
+      const bf16_t* krow = Ks + col * KS + 8 * half;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s) {
+        const bf16x8v a = *reinterpret_cast<const bf16x8v*>(krow + 16 * s);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qh[s], S, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qm[s], S, 0, 0, 0);
+        S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, ql[s], S, 0, 0, 0);
+      }
+    }
+    // ---- mask, soft cap, weights (column = query, 16 keys in-lane) ---------------
+    const int jt0 = lo + u0;
+    const bool interior = nq == RM_Q && u0 + RM_K <= nk && jt0 + RM_K - 1 <= p0 &&
+                          (window == 0 || p_last - jt0 < window);
+    float corr = 1.f;
+    if (SIG) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int u = u0 + 8 * i + 4 * half + j;
+          const int jt = lo + u;
+          const bool vis = interior || (jt <= pq && (window == 0 || pq - jt < window) &&
+                                        qvalid && u < nk);
+          float sc = S[4 * i + j] * scale;
+          if (softcap > 0.f) sc = softcap * rm_tanh(sc * inv_cap);
+          S[4 * i + j] = vis ? rm_sigmoid(sc + hbias) : 0.f;
+        }
+    } else {
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int u = u0 + 8 * i + 4 * half + j;
+          const int jt = lo + u;
+          const bool vis = interior || (jt <= pq && (window == 0 || pq - jt < window) &&
+                                        qvalid && u < nk);
+          float sc = S[4 * i + j] * scale;
+          if (softcap > 0.f) sc = softcap * rm_tanh(sc * inv_cap);
+          sc = vis ? sc : -INFINITY;
+          S[4 * i + j] = sc;
+          tmax = fmaxf(tmax, sc);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(mx, tmax);
+      float psum = 0.f;
+      if (m_new == -INFINITY) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) S[i] = 0.f;
+      } else {
+        corr = __expf(mx - m_new);  // exp(-inf) = 0 the first time a key is seen
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float p = __expf(S[i] - m_new);  // exp(-inf) = 0 for masked keys
+          S[i] = p;
+          psum += p;
+        }
+      }
+      psum += __shfl_xor(psum, 32, 64);
+      l = l * corr + psum;
+      mx = m_new;
+#pragma unroll
+      for (int k = 0; k < DVB; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[k][i] *= corr;
+    }
+    // ---- O^T += V_tile^T . P^T, three parts of p ---------------------------------
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      bf16x8v ph, pm, pl;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        short a, m, lw;
+        rb_split3(S[8 * s + e], a, m, lw);
+        ph[e] = a;
+        pm[e] = m;
+        pl[e] = lw;
+      }
+#pragma unroll
+      for (int k = 0; k < DVB; ++k) {
+        const bf16_t* vrow = Vt + (32 * k + col) * RB_VS + 16 * s + 4 * half;
+        const int2 v0 = *reinterpret_cast<const int2*>(vrow);
+        const int2 v1 = *reinterpret_cast<const int2*>(vrow + 8);
+        const int4 packed = make_int4(v0.x, v0.y, v1.x, v1.y);
+        const bf16x8v a = *reinterpret_cast<const bf16x8v*>(&packed);
+        acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, ph, acc[k], 0, 0, 0);
+        acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pm, acc[k], 0, 0, 0);
+        acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pl, acc[k], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- epilogue: lane holds O[query col][feature 32 k + 8 i + 4 half + j] --------
+  const float inv = SIG ? (qvalid ? 1.0f : 0.f)
+                        : ((qvalid && l > 0.f) ? 1.0f / l : 0.f);
+#pragma unroll
+  for (int k = 0; k < DVB; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[k][i] *= inv;
+  if (rot_cs != nullptr) {
+    const float* rc = rot_cs + (int64_t)(t0 + min(col, nq - 1)) * dv;
+    if (rot_inter) {
+#pragma unroll
+      for (int k = 0; k < DVB; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+          const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+          if (f < dv) {
+            const float2 cs = *reinterpret_cast<const float2*>(rc + f);
+            const float u = acc[k][i], w = acc[k][i + 1];
+            acc[k][i] = fmaf(w, cs.y, u * cs.x);
+            acc[k][i + 1] = fmaf(-u, cs.y, w * cs.x);
+          }
+        }
+    } else {
+#pragma unroll
+      for (int k = 0; k < DVB / 2; ++k)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+          const float2 cs = *reinterpret_cast<const float2*>(rc + 2 * f);
+          const float u = acc[k][i], w = acc[k + DVB / 2][i];
+          acc[k][i] = fmaf(w, cs.y, u * cs.x);
+          acc[k + DVB / 2][i] = fmaf(-u, cs.y, w * cs.x);
+        }
+    }
+  }
+  float r = 1.0f;
+  if (norm_eps >= 0.f) {
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < DVB; ++k)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ss += acc[k][i] * acc[k][i];
+    ss += __shfl_xor(ss, 32, 64);
+    r = out_mult / sqrtf(ss / (float)dv + norm_eps);
+  }
+  if (!stream_on || !qvalid) return;
+  if (gate != nullptr)
+    r *= rm_sigmoid_exact(ldf(gate + (int64_t)(t0 + col) * gate_stride + h));
+  const int64_t o0 = ((int64_t)(t0 + col) * H + h) * dv;
+#pragma unroll
+  for (int k = 0; k < DVB; ++k)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int f = 32 * k + 8 * (i >> 2) + 4 * half + (i & 3);
+      if (f < dv) {
+        if (out32 != nullptr) out32[o0 + f] = acc[k][i] * r;
+        else stf(out + o0 + f, acc[k][i] * r);
+      }
+    }
+}
+
 struct RmArgs {
   void* out;
   float* out32;
@@ -514,9 +837,41 @@ struct RmArgs {
   hipStream_t stream;
 };
 
+// PARALLAX_ROW_ATTN_FP32=1 keeps bf16 rows on the fp32 matrix cores too
+static bool rm_split_bf16() {
+  static const bool on = []() {
+    const char* e = getenv("PARALLAX_ROW_ATTN_FP32");
+    return !(e && e[0] == '1');
+  }();
+  return on;
+}
+
+template <int D, int DVB, bool SIG>
+static void launch_rb(const RmArgs& a) {
+  constexpr int DV = DVB * 32;
+  const int rep = a.H / a.G;
+  const size_t shm = sizeof(bf16_t) * ((size_t)RM_K * (D + RB_KPAD) + (size_t)DV * RB_VS);
+  const dim3 grid(a.tiles, a.G * ((rep + 3) / 4));
+  hipLaunchKernelGGL((row_attention_prefill_bf16_kernel<D, DVB, SIG>), grid,
+                     dim3(256), shm, a.stream, (bf16_t*)a.out, a.out32, a.q,
+                     (const bf16_t*)a.cache, a.block_tables, a.bt_stride, a.cu,
+                     a.B, a.positions, a.H, a.G, a.d, a.dv, a.block_size,
+                     a.window, a.scale, a.softcap, a.norm_eps, a.out_mult,
+                     a.head_bias, (const bf16_t*)a.gate, a.gate_stride, a.vbase,
+                     a.rot_cs, a.rot_inter);
+}
+
 template <typename T, int M, int D, int DVB, bool SIG>
 static void launch_rm_k(const RmArgs& a) {
   constexpr int DV = DVB * 32;
+  // bf16 rows, one score map, no pooled rows, value tiles up to 128: the
+  // exact three-part products on the bf16 matrix cores
+  if constexpr (std::is_same<T, bf16_t>::value && M == 1 && DVB <= 4) {
+    if (a.P == 0 && rm_split_bf16()) {
+      launch_rb<D, DVB, SIG>(a);
+      return;
+    }
+  }
   const int rep = a.H / a.G;
   const int hw = 4 / M;
   const size_t stage = (size_t)M * RM_K * (D + RM_PAD) + RM_K * (DV + RM_PAD);
