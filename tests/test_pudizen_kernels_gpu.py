@@ -194,3 +194,45 @@ def test_rows_whose_values_are_their_keys(dt, H, r):
                                     query_bounds=bounds.to(DEV) if tiled else None,
                                     gate=gate.to(DEV), shared_kv=True, value_col=c0)
             assert close(got, want, 2e-5), (tiled, "share")
+
+
+@pytest.mark.parametrize("H,G,d,dv,win,sig", [
+    (8, 2, 128, 128, 0, False),
+    (4, 4, 64, 64, 200, True),
+    (6, 1, 40, 96, 0, True),
+    (3, 3, 128, 32, 333, False),
+])
+def test_three_part_bf16_products_are_exact(H, G, d, dv, win, sig):
+    """Prompt portions over bf16 rows run both products on the bf16 matrix
+    cores with the fp32 operand split into three bf16 parts: the result must
+    equal the fp32 arithmetic of the reference (and of the per-token kernel)
+    to rounding, over many key steps, ragged tiles and portions that start
+    in the middle of a sequence."""
+    g = torch.Generator().manual_seed(d + dv)
+    bs, nblk = 32, 40
+    lens = [700, 45, 290]
+    starts = [0, 13, 258]           # the portions' first positions
+    pos = torch.cat([torch.arange(s0, n) for s0, n in zip(starts, lens)]).int()
+    seq = torch.cat([torch.full((n - s0,), i) for i, (s0, n) in enumerate(zip(starts, lens))]).int()
+    T = pos.numel()
+    perm = torch.randperm(nblk, generator=g)
+    bt = torch.zeros(3, 22, dtype=torch.int32)
+    o = 0
+    for i, n in enumerate(lens):
+        nb = (n + bs - 1) // bs
+        bt[i, :nb] = perm[o:o + nb]
+        o += nb
+    bounds = torch.tensor([0] + torch.tensor([n - s0 for s0, n in zip(starts, lens)])
+                          .cumsum(0).tolist(), dtype=torch.int32)
+    cache = (torch.randn(nblk, bs, G * d + G * dv, generator=g) * 0.7).to(torch.bfloat16)
+    q = torch.randn(T, H * d, generator=g) * 1.3
+    bias = torch.randn(H, generator=g) - 3 if sig else None
+    want = ref.row_attention(q, cache, None, bt, seq, pos, H, G, 1, d, dv, win, 0, d ** -0.5,
+                             0.0, 0.0, None, 1.0, torch.float32, bias)
+    for tiled in (True, False):
+        got = ops.row_attention(q.to(DEV), cache.to(DEV), None, bt.to(DEV), seq.to(DEV),
+                                pos.to(DEV), H, G, 1, d, dv, win, 0, d ** -0.5, 0.0, 0.0, None,
+                                1.0, torch.float32, max_seq_len=max(lens),
+                                query_bounds=bounds.to(DEV) if tiled else None,
+                                head_bias=gpu(bias))
+        assert close(got, want, 3e-5), tiled
