@@ -322,6 +322,8 @@ PUDIZEN_SIZES = {
               window=512, rank=128, vocab=32000),
     "m": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=8192,
               window=1024, rank=128, vocab=32000),
+    "l": dict(width=4096, layers=8, heads=32, kv_heads=8, dim=128, ff=14336,
+              window=1024, rank=128, vocab=32000),
 }
 
 # layer kinds of the stack, repeated: window, latent, window, softmax
@@ -496,7 +498,8 @@ def main():
                          "Qwen3-MoE-style stack, or pudizen beside a "
                          "Qwen3-style dense stack")
     ap.add_argument("--design-sizes", default="s,m",
-                    help="comma list of " + ",".join(DESIGN_SIZES))
+                    help="comma list of " + ",".join(DESIGN_SIZES)
+                    + " (the pudizen pair also has l)")
     ap.add_argument("--design-batch", type=int, default=8)
     ap.add_argument("--design-prompt", type=int, default=2048)
     ap.add_argument("--design-only", default="",
